@@ -1,4 +1,5 @@
 from .model_config import ConfigError, Qwen3Config, read_config_json, FULL_ATTENTION, SLIDING_ATTENTION
+from .visadra_config import VisadraConfig
 from .registry import (
     Architecture,
     architecture_of,
@@ -12,6 +13,7 @@ __all__ = [
     "Architecture",
     "ConfigError",
     "Qwen3Config",
+    "VisadraConfig",
     "FULL_ATTENTION",
     "SLIDING_ATTENTION",
     "architecture_of",

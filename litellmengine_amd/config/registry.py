@@ -48,9 +48,12 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_of(config_dict: Dict[str, Any]) -> Architecture:
     archs = config_dict.get("architectures")
-    if not archs or not isinstance(archs, list):
-        raise ConfigError("config.json has no `architectures` list to choose a model by")
-    return get_architecture(str(archs[0]))
+    if archs and isinstance(archs, list):
+        return get_architecture(str(archs[0]))
+    one = config_dict.get("architecture")  # some families name themselves with one string
+    if isinstance(one, str) and one:
+        return get_architecture(one)
+    raise ConfigError("config.json has no `architectures` list (or `architecture` name) to choose a model by")
 
 
 def architecture_of_model_dir(model_dir: str) -> Architecture:

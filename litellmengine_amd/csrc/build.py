@@ -32,6 +32,9 @@ LIBRARIES: Dict[str, List[str]] = {
     "attention": ["attention.hip"],
     "gemm": ["gemm.hip"],
     "sampling": ["sampling.hip"],
+    "recurrent": ["recurrent.hip"],
+    "latent": ["latent.hip"],
+    "moe": ["moe.hip"],
     "probe": ["probe.hip"],
 }
 # libraries without GPU code: compiled with the host's C++ compiler

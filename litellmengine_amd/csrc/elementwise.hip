@@ -15,7 +15,7 @@ LLE_DEFINE_ERROR_STRING()
 template <typename T>
 __global__ __launch_bounds__(256) void embedding_kernel(const int32_t* __restrict__ ids,
                                                          const T* __restrict__ table,
-                                                         float* __restrict__ out, int H,
+                                                         float* __restrict__ out, int H, float scale,
                                                          const int32_t* __restrict__ feedback,
                                                          const int32_t* __restrict__ token_seq,
                                                          const int32_t* __restrict__ seq_slots) {
@@ -24,25 +24,31 @@ __global__ __launch_bounds__(256) void embedding_kernel(const int32_t* __restric
     if (id < 0) id = feedback ? feedback[seq_slots[token_seq[n]]] : 0;
     const T* row = table + (int64_t)id * H;
     float* o = out + n * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<T>(row[i]);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<T>(row[i]) * scale;  // (times 1 is exact)
 }
 
-// `feedback`, `token_seq` [N] and `seq_slots`: all three or none
-extern "C" int lle_embedding_feedback(const void* ids, const void* table, void* out, int N, int H, int dtype,
-                                      const void* feedback, const void* token_seq, const void* seq_slots,
-                                      hipStream_t stream) {
+// `feedback`, `token_seq` [N] and `seq_slots`: all three or none; every row is multiplied by `scale` in 32-bit
+extern "C" int lle_embedding_scaled(const void* ids, const void* table, void* out, int N, int H, int dtype,
+                                    const void* feedback, const void* token_seq, const void* seq_slots, float scale,
+                                    hipStream_t stream) {
     if (N <= 0) return 0;
     if ((feedback != nullptr) != (token_seq != nullptr) || (feedback != nullptr) != (seq_slots != nullptr))
         return (int)hipErrorInvalidValue;
     if (dtype == LLE_F32)
-        embedding_kernel<float><<<N, 256, 0, stream>>>((const int32_t*)ids, (const float*)table, (float*)out, H,
+        embedding_kernel<float><<<N, 256, 0, stream>>>((const int32_t*)ids, (const float*)table, (float*)out, H, scale,
                                                         (const int32_t*)feedback, (const int32_t*)token_seq,
                                                         (const int32_t*)seq_slots);
     else
-        embedding_kernel<bf16_t><<<N, 256, 0, stream>>>((const int32_t*)ids, (const bf16_t*)table, (float*)out, H,
+        embedding_kernel<bf16_t><<<N, 256, 0, stream>>>((const int32_t*)ids, (const bf16_t*)table, (float*)out, H, scale,
                                                          (const int32_t*)feedback, (const int32_t*)token_seq,
                                                          (const int32_t*)seq_slots);
     LLE_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int lle_embedding_feedback(const void* ids, const void* table, void* out, int N, int H, int dtype,
+                                      const void* feedback, const void* token_seq, const void* seq_slots,
+                                      hipStream_t stream) {
+    return lle_embedding_scaled(ids, table, out, N, H, dtype, feedback, token_seq, seq_slots, 1.0f, stream);
 }
 
 extern "C" int lle_embedding(const void* ids, const void* table, void* out, int N, int H, int dtype,
@@ -124,5 +130,43 @@ extern "C" int lle_add_bias(void* x, const void* bias, int M, int N, int dtype, 
     else if (bias_dtype == LLE_F32) LLE_BIAS_CASE(bf16_t, float);
     else LLE_BIAS_CASE(bf16_t, bf16_t);
 #undef LLE_BIAS_CASE
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// out = x in another float type (the rows of the 32-bit residual stream for a sublayer that reads them)
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void cast_kernel(const TI* __restrict__ x, TO* __restrict__ out, int64_t total) {
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x)
+        out[idx] = from_f32<TO>(to_f32<TI>(x[idx]));
+}
+
+extern "C" int lle_cast(const void* x, void* out, int64_t total, int in_dtype, int out_dtype, hipStream_t stream) {
+    if (total <= 0) return 0;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (in_dtype == LLE_F32 && out_dtype == LLE_BF16)
+        cast_kernel<float, bf16_t><<<(int)blocks, 256, 0, stream>>>((const float*)x, (bf16_t*)out, total);
+    else if (in_dtype == LLE_BF16 && out_dtype == LLE_F32)
+        cast_kernel<bf16_t, float><<<(int)blocks, 256, 0, stream>>>((const bf16_t*)x, (float*)out, total);
+    else if (in_dtype == LLE_F32)
+        cast_kernel<float, float><<<(int)blocks, 256, 0, stream>>>((const float*)x, (float*)out, total);
+    else
+        cast_kernel<bf16_t, bf16_t><<<(int)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, total);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// x *= factor in place, float32 (the logits of a model that scales them)
+__global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ x, int64_t total, float factor) {
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x)
+        x[idx] *= factor;
+}
+
+extern "C" int lle_scale(void* x, int64_t total, float factor, hipStream_t stream) {
+    if (total <= 0) return 0;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    scale_kernel<<<(int)blocks, 256, 0, stream>>>((float*)x, total, factor);
     LLE_RETURN_LAUNCH_STATUS();
 }

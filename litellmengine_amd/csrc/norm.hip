@@ -328,3 +328,46 @@ extern "C" int lle_rmsnorm(const void* x, const void* weight, int weight_dtype, 
         rmsnorm_kernel<bf16_t><<<R, 256, 0, stream>>>((const bf16_t*)x, weight, weight_dtype, (bf16_t*)out, H, eps);
     LLE_RETURN_LAUNCH_STATUS();
 }
+
+// For arrangements that norm a sublayer's OUTPUT: hidden[r] += norm(y[r] (+ extra[r])) * w, in 32-bit and in
+// place, and the new row of `hidden` leaves in the activation type TO as well (the next sublayer reads it).
+// `y` and `extra` hold float32 or bfloat16, each said by its own code.
+template <typename TO>
+__global__ __launch_bounds__(1024) void rmsnorm_add_kernel(float* __restrict__ hidden, const void* __restrict__ y,
+                                                            int y_dtype, const void* __restrict__ extra,
+                                                            int extra_dtype, const void* __restrict__ weight,
+                                                            int weight_dtype, TO* __restrict__ out, int H, float eps) {
+    __shared__ float red[16];
+    const int64_t r = blockIdx.x;
+    const int64_t at = r * H;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = load_as_f32(y, at + i, y_dtype);
+        if (extra) v += load_as_f32(extra, at + i, extra_dtype);
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = load_as_f32(y, at + i, y_dtype);
+        if (extra) v += load_as_f32(extra, at + i, extra_dtype);
+        const float h = hidden[at + i] + v * inv * load_as_f32(weight, i, weight_dtype);
+        hidden[at + i] = h;
+        if (out) out[at + i] = from_f32<TO>(h);
+    }
+}
+
+// `out` may be null (float32 callers read `hidden` itself)
+extern "C" int lle_rmsnorm_add(void* hidden, const void* y, int y_dtype, const void* extra, int extra_dtype,
+                               const void* weight, int weight_dtype, void* out, int R, int H, float eps,
+                               int out_dtype, hipStream_t stream) {
+    if (R <= 0) return 0;
+    const int threads = H > 8192 ? 1024 : H > 2048 ? 512 : 256;
+    if (out_dtype == LLE_F32)
+        rmsnorm_add_kernel<float><<<R, threads, 0, stream>>>((float*)hidden, y, y_dtype, extra, extra_dtype, weight,
+                                                              weight_dtype, (float*)out, H, eps);
+    else
+        rmsnorm_add_kernel<bf16_t><<<R, threads, 0, stream>>>((float*)hidden, y, y_dtype, extra, extra_dtype, weight,
+                                                               weight_dtype, (bf16_t*)out, H, eps);
+    LLE_RETURN_LAUNCH_STATUS();
+}

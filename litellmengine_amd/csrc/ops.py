@@ -98,8 +98,8 @@ class HipOps:
 
     # -- embedding -----------------------------------------------------------
     def embedding(self, ids: torch.Tensor, table: torch.Tensor, feedback=None, token_seq=None,
-                  seq_slots=None) -> torch.Tensor:
-        """ids int32 [N], table [V, H] -> float32 [N, H] (the residual stream).  With `feedback`
+                  seq_slots=None, scale: float = 1.0) -> torch.Tensor:
+        """ids int32 [N], table [V, H] -> float32 [N, H] (the residual stream), times `scale`.  With `feedback`
         (int32, indexed by request slot), `token_seq` [N] and `seq_slots`: an id below zero is
         replaced by feedback[seq_slots[token_seq[n]]], the token that argmax(..., scatter=...) left there."""
         _dev(ids, "ids", torch.int32)
@@ -112,9 +112,10 @@ class HipOps:
                 _dev(t, name, torch.int32)
             _need(token_seq.shape == (N,), "token_seq must be [N]")
         out = torch.empty((N, H), dtype=torch.float32, device=table.device)
-        self._run("elementwise", "lle_embedding_feedback", [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P],
+        self._run("elementwise", "lle_embedding_scaled", [_P, _P, _P, _I, _I, _I, _P, _P, _P, _F, _P],
                   _ptr(ids), _ptr(table), _ptr(out), N, H, dtype_code(table.dtype), _ptr(feedback),
-                  _ptr(token_seq) if feedback is not None else None, _ptr(seq_slots) if feedback is not None else None)
+                  _ptr(token_seq) if feedback is not None else None, _ptr(seq_slots) if feedback is not None else None,
+                  float(scale))
         return out
 
     def embedding_rmsnorm(self, ids, table, weight, eps: float, feedback=None, token_seq=None, seq_slots=None):
@@ -679,6 +680,198 @@ class HipOps:
                       _ptr(x), _ptr(weight), _ptr(out), M, N2, K)
             return out
         return self.silu_mul(self.linear(x, weight))
+
+    # -- arrangements that norm a sublayer's output ------------------------------------
+    def cast(self, x, dtype) -> torch.Tensor:
+        """x in `dtype` (x itself where it has that type already)."""
+        if x.dtype == dtype:
+            return x
+        _dev(x, "x")
+        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+        self._run("elementwise", "lle_cast", [_P, _P, _L, _I, _I, _P], _ptr(x), _ptr(out), x.numel(),
+                  dtype_code(x.dtype), dtype_code(dtype))
+        return out
+
+    def scale_(self, x, factor: float) -> torch.Tensor:
+        """float32 x *= factor, in place."""
+        _dev(x, "x", torch.float32)
+        self._run("elementwise", "lle_scale", [_P, _L, _F, _P], _ptr(x), x.numel(), float(factor))
+        return x
+
+    def rmsnorm_add(self, hidden, y, weight, eps: float, out_dtype, extra=None) -> torch.Tensor:
+        """hidden float32 [N, H] += RMSNorm(y [+ extra]) * weight, in place and in 32-bit; returns the new
+        rows in `out_dtype` (`hidden` itself for float32).  `y`, `extra`: [N, H], float32 or bfloat16 each."""
+        _dev(hidden, "hidden", torch.float32)
+        _dev(weight, "norm weight")
+        N, H = hidden.shape
+        _need(weight.shape == (H,), f"norm weight must be [{H}], is {list(weight.shape)}")
+        for t, name in ((y, "y"), (extra, "extra")):
+            if t is not None:
+                _dev(t, name)
+                _need(t.shape == hidden.shape, f"{name} must have the shape of hidden")
+        out = None if out_dtype == torch.float32 else torch.empty((N, H), dtype=out_dtype, device=hidden.device)
+        self._run("norm", "lle_rmsnorm_add", [_P, _P, _I, _P, _I, _P, _I, _P, _I, _I, _F, _I, _P],
+                  _ptr(hidden), _ptr(y), dtype_code(y.dtype), _ptr(extra), dtype_code(extra.dtype) if extra is not None else 0,
+                  _ptr(weight), dtype_code(weight.dtype), _ptr(out), N, H, float(eps), dtype_code(out_dtype))
+        return hidden if out is None else out
+
+    # -- gated recurrence -------------------------------------------------------------
+    MINGRU_PIECE = 64  # tokens of one request that one thread walks before the walk is cut into pieces
+
+    def mingru_scan(self, zxg, z_bias, x_bias, state, seq_slots, cu_tokens, out_dtype, max_q_len: int = 0):
+        """zxg [N, 3 W] (update-gate, candidate and output-gate inputs side by side; float32 or bfloat16),
+        biases float32 [W], state float32 [slots + 1, W] (read and advanced per request) -> [N, W] in
+        `out_dtype`: S <- (1 - z) S + z c per token, out = S * silu(gate).  `max_q_len` (a host-side
+        bound of the longest request of the step) only decides into how many pieces a walk is cut."""
+        _dev(zxg, "zxg")
+        _dev(z_bias, "z_bias", torch.float32)
+        _dev(x_bias, "x_bias", torch.float32)
+        _dev(state, "state", torch.float32)
+        _dev(seq_slots, "seq_slots", torch.int32)
+        _dev(cu_tokens, "cu_tokens", torch.int32)
+        W = z_bias.shape[0]
+        N, S = zxg.shape[0], seq_slots.shape[0]
+        _need(zxg.shape == (N, 3 * W) and x_bias.shape == (W,), "zxg must be [N, 3 W] and the biases [W]")
+        _need(state.dim() == 2 and state.shape[1] == W, "state must be [slots, W]")
+        _need(cu_tokens.shape == (S + 1,), "cu_tokens must be [S + 1]")
+        out = torch.empty((N, W), dtype=out_dtype, device=zxg.device)
+        pieces = max(1, min(1024, -(-max(1, max_q_len) // self.MINGRU_PIECE)))
+        part = torch.empty((S * pieces * 2 * W,), dtype=torch.float32, device=zxg.device) if pieces > 1 else None
+        self._run("recurrent", "lle_mingru_scan", [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _P],
+                  _ptr(zxg), dtype_code(zxg.dtype), _ptr(z_bias), _ptr(x_bias), _ptr(state), _ptr(seq_slots),
+                  _ptr(cu_tokens), _ptr(out), dtype_code(out_dtype), _ptr(part), S, W, pieces)
+        return out
+
+    # -- latent attention -------------------------------------------------------------
+    def latent_kv_write(self, dkv, norm_w, eps: float, cos_sin, rot_dims: int, slots, pages, page_size: int,
+                        rank: int, rot: int) -> None:
+        """dkv [N, rank + rot] -> the pages: c = RMSNorm(first rank) * norm_w and the rest with its first
+        `rot_dims` elements rotated in neighbouring pairs by cos_sin [N, rot_dims / 2, 2].  A page
+        (one row of `pages`) is [page_size][rank] then [page_size][rot]; slots[n] < 0 writes nothing."""
+        _dev(dkv, "dkv")
+        _dev(norm_w, "latent norm weight")
+        _dev(slots, "slots", torch.int32)
+        N = dkv.shape[0]
+        _need(dkv.shape == (N, rank + rot) and norm_w.shape == (rank,) and slots.shape == (N,), "dkv [N, rank + rot]")
+        _need(pages.is_cuda and pages.dtype == dkv.dtype and pages.dim() == 2 and pages.stride(1) == 1
+              and pages.shape[1] >= page_size * (rank + rot), "pages must be [pages, page_size * (rank + rot)]")
+        if rot_dims:
+            _dev(cos_sin, "cos_sin", torch.float32)
+            _need(cos_sin.shape == (N, rot_dims // 2, 2), "cos_sin must be [N, rot_dims / 2, 2]")
+        self._run("latent", "lle_latent_kv_write", [_P, _P, _I, _F, _P, _I, _P, _P, _L, _I, _I, _I, _I, _I, _P],
+                  _ptr(dkv), _ptr(norm_w), dtype_code(norm_w.dtype), float(eps), _ptr(cos_sin) if rot_dims else None,
+                  int(rot_dims), _ptr(slots), _ptr(pages), pages.stride(0), int(page_size), N, rank, rot,
+                  dtype_code(dkv.dtype))
+
+    def latent_q_rope(self, q, cos_sin, rot_dims: int, heads: int, dim: int, rot: int) -> torch.Tensor:
+        """q [N, heads * (dim + rot)] -> the last `rot` elements of every head, rotated, float32 [N, heads, rot]."""
+        _dev(q, "q")
+        N = q.shape[0]
+        _need(q.shape == (N, heads * (dim + rot)), "q must be [N, heads * (dim + rot)]")
+        if rot_dims:
+            _dev(cos_sin, "cos_sin", torch.float32)
+            _need(cos_sin.shape == (N, rot_dims // 2, 2), "cos_sin must be [N, rot_dims / 2, 2]")
+        out = torch.empty((N, heads, rot), dtype=torch.float32, device=q.device)
+        self._run("latent", "lle_latent_q_rope", [_P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+                  _ptr(q), _ptr(cos_sin) if rot_dims else None, int(rot_dims), _ptr(out), N, heads, dim, rot,
+                  dtype_code(q.dtype))
+        return out
+
+    def heads_linear(self, x, heads: int, col0: int, K: int, weight, out_dtype) -> torch.Tensor:
+        """x [N, heads * xw] (or [N, heads, xw]) and weight [heads, out, K]: for every head the columns
+        col0 .. col0 + K of its part times weight[h]^T -> [N, heads, out].  bfloat16: one batched
+        library product (32-bit accumulation, either result type); float32: the true 32-bit kernels, head by head."""
+        _dev(x, "x")
+        _dev(weight, "weight", x.dtype)
+        N = x.shape[0]
+        x3 = x.view(N, heads, -1)
+        xw, O = x3.shape[2], weight.shape[1]
+        _need(weight.shape == (heads, O, K) and 0 <= col0 and col0 + K <= xw, "weight must be [heads, out, K]")
+        if x.dtype == torch.bfloat16:
+            a = x3[:, :, col0 : col0 + K].transpose(0, 1)  # [heads, N, K]
+            b = weight.transpose(1, 2)  # [heads, K, out]
+            y = torch.bmm(a, b) if out_dtype == torch.bfloat16 else torch.bmm(a, b, out_dtype=out_dtype)
+            return y.transpose(0, 1)  # [N, heads, out], strided
+        _need(out_dtype == torch.float32, "a float32 product has a float32 result")
+        out = torch.empty((N, heads, O), dtype=torch.float32, device=x.device)
+        quick = K % 4 == 0 and xw % 4 == 0 and col0 % 4 == 0 and not self.force_simt_gemm
+        for h in range(heads):
+            a_ptr = x.data_ptr() + 4 * (h * xw + col0)
+            b_ptr = weight.data_ptr() + 4 * h * O * K
+            c_ptr = out.data_ptr() + 4 * h * O
+            if quick:
+                self._run("gemm", "lle_gemm_nt_mfma_f32", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _P],
+                          a_ptr, b_ptr, c_ptr, N, O, K, heads * xw, K, heads * O)
+            else:
+                self._run("gemm", "lle_gemm_nt_simt", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _I, _P],
+                          a_ptr, b_ptr, c_ptr, N, O, K, heads * xw, K, heads * O, F32, F32)
+        return out
+
+    def latent_attention(self, q_lat, q_rot, pages, page_size: int, rank: int, rot: int, block_table, seq_slots,
+                         cu_tokens, kv_lens, token_seq, sink, window: Optional[int], scale: float, max_q_len: int,
+                         max_kv_len: int, out_dtype) -> torch.Tensor:
+        """All heads of every token against the cached latents: q_lat [N, H, rank] (float32 or the
+        cache's type; any strides over N and H), q_rot float32 [N, H, rot], sink float32 [H] ->
+        sum_j p_j c_j, [N, H, rank] in the cache's type.  `max_q_len` and `max_kv_len` are host-side
+        bounds; they choose kernels, never results."""
+        _dev(q_rot, "q_rot", torch.float32)
+        _dev(sink, "sink", torch.float32)
+        for t, name in ((block_table, "block_table"), (seq_slots, "seq_slots"), (cu_tokens, "cu_tokens"),
+                        (kv_lens, "kv_lens"), (token_seq, "token_seq")):
+            _dev(t, name, torch.int32)
+        N, H, _ = q_lat.shape
+        S = seq_slots.shape[0]
+        _need(q_lat.is_cuda and q_lat.shape == (N, H, rank) and q_lat.stride(2) == 1, "q_lat must be [N, H, rank]")
+        _need(q_lat.dtype in (torch.float32, pages.dtype), "q_lat is float32 or of the cache's type")
+        _need(q_rot.shape == (N, H, rot) and sink.shape == (H,), "q_rot [N, H, rot], sink [H]")
+        _need(pages.is_cuda and pages.dim() == 2 and pages.stride(1) == 1 and pages.dtype == out_dtype
+              and pages.shape[1] >= page_size * (rank + rot), "pages must be [pages, page_size * (rank + rot)]")
+        _need(token_seq.shape == (N,) and cu_tokens.shape == (S + 1,) and kv_lens.shape == (S,), "the step's arrays")
+        _need(block_table.dim() == 2, "block_table must be [slots, pages]")
+        _need(rank <= 1024, f"a latent of {rank} elements is wider than the attention kernels take (1024)")
+        out = torch.empty((N, H, rank), dtype=out_dtype, device=pages.device)
+        self._run("latent", "lle_latent_attention_generic",
+                  [_P, _I, _L, _L, _P, _P, _L, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _F, _P, _I, _I, _I, _P],
+                  _ptr(q_lat), dtype_code(q_lat.dtype), q_lat.stride(0), q_lat.stride(1), _ptr(q_rot), _ptr(pages),
+                  pages.stride(0), int(page_size), rank, rot, _ptr(block_table), block_table.shape[1], _ptr(seq_slots),
+                  _ptr(cu_tokens), _ptr(kv_lens), _ptr(token_seq), _ptr(sink), int(window) if window else 0,
+                  float(scale), _ptr(out), N, H, dtype_code(out_dtype))
+        return out
+
+    # -- routed feed-forward ----------------------------------------------------------
+    def moe_route(self, logits, bias, top: int):
+        """float32 logits [N, E] + bias [E] -> (int32 ids [N, top] of the largest, the lower index first
+        among equals; float32 gains [N, top]: the softmax over the chosen alone)."""
+        _dev(logits, "router logits", torch.float32)
+        _dev(bias, "router bias", torch.float32)
+        N, E = logits.shape
+        _need(bias.shape == (E,) and 0 < top <= min(E, 16), "a router picks between 1 and 16 of its experts")
+        ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
+        gains = torch.empty((N, top), dtype=torch.float32, device=logits.device)
+        self._run("moe", "lle_moe_route", [_P, _P, _P, _P, _I, _I, _I, _P], _ptr(logits), _ptr(bias), _ptr(ids),
+                  _ptr(gains), N, E, top)
+        return ids, gains
+
+    def moe_experts(self, x, ids, gains, gate_up, down) -> torch.Tensor:
+        """x [N, K]; ids, gains [N, top]; gate_up [E, 2 F, K] (gate rows, then up rows); down [E, H, F] ->
+        float32 [N, H]: sum_k gains[n, k] * down[e] (silu(gate[e] x) * (up[e] x)), e = ids[n, k]."""
+        _dev(x, "x")
+        _dev(ids, "ids", torch.int32)
+        _dev(gains, "gains", torch.float32)
+        _dev(gate_up, "gate_up", x.dtype)
+        _dev(down, "down", x.dtype)
+        N, K = x.shape
+        top = ids.shape[1]
+        E, F2, _ = gate_up.shape
+        H = down.shape[1]
+        _need(ids.shape == (N, top) and gains.shape == (N, top), "ids and gains must be [N, top]")
+        _need(gate_up.shape == (E, F2, K) and F2 % 2 == 0 and down.shape == (E, H, F2 // 2), "expert weights do not fit")
+        act = torch.empty((N * top, F2 // 2), dtype=x.dtype, device=x.device)
+        out = torch.empty((N, H), dtype=torch.float32, device=x.device)
+        self._run("moe", "lle_moe_experts", [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+                  _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(act), _ptr(out), N, top, F2 // 2,
+                  K, H, dtype_code(x.dtype))
+        return out
 
     # -- picking tokens --------------------------------------------------------------
     def argmax(self, logits, scatter=None) -> torch.Tensor:

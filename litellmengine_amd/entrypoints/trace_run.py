@@ -33,7 +33,7 @@ def parse_args(argv=None):
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens the live requests hold at any time (each rounded up to 64)")
     p.add_argument("--page-size", type=int, default=16)
-    p.add_argument("--max-requests", type=int, default=16, help="request slots")
+    p.add_argument("--max-requests", type=int, default=4, help="request slots (and state rows): most requests alive at once")
     return p.parse_args(argv)
 
 

@@ -1,4 +1,5 @@
 from . import qwen3  # noqa: F401  (registers Qwen3ForCausalLM)
+from . import visadra  # noqa: F401  (registers Visadra)
 from .build import expected_tensors, load_model, make_context, parse_dtype, random_model
 from .decoder import DecoderLM, PlanEntry
 

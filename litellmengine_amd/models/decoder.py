@@ -16,7 +16,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import Block, BuildContext, Norm, Prenormed
+from ..parts.base import Block, BuildContext, Carried, Norm, Prenormed
 from ..parts.embedding import Embedding
 from ..parts.linear import Linear
 from ..weights.spec import TensorSpec
@@ -43,7 +43,10 @@ class DecoderLM:
         final_norm: Norm,
         head: Linear,
         tied_head: bool,
+        logit_scale: float = 1.0,
     ):
+        """`logit_scale`: the head's result is multiplied by it (in 32-bit)."""
+        self.logit_scale = float(logit_scale)
         self.config = config
         self.embedding = embedding
         self.blocks = list(blocks)
@@ -119,5 +122,8 @@ class DecoderLM:
             delta = self.blocks[e.block].forward(hidden, delta, step, caches.layer(i), next_norm=next_norm)
         if step.logit_rows.shape[0] == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=hidden.device)
+        if isinstance(delta, Carried):  # the last block has added everything into the stream itself
+            delta = None
         x = delta if isinstance(delta, Prenormed) else self.final_norm.forward(hidden, delta, rows=step.logit_rows)
-        return self.head.forward(x, out_dtype=torch.float32)
+        logits = self.head.forward(x, out_dtype=torch.float32)
+        return logits if self.logit_scale == 1.0 else self.ctx.ops.scale_(logits, self.logit_scale)

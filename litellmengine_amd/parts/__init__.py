@@ -1,15 +1,19 @@
 from .attention import PagedAttention
-from .base import (Block, BuildContext, CacheField, CacheSpec, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part,
+from .base import (Block, BuildContext, CacheField, Carried, CacheSpec, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part,
                    Normed, PartialSums, PositionEncoding, Prenormed, StateSpec)
-from .block import PreNormBlock
+from .block import PostNormBlock, PreNormBlock
 from .embedding import Embedding
 from .feed_forward import GatedMLP
+from .latent_attention import LatentAttention
 from .linear import Linear
+from .moe import RoutedMLP
 from .norm import RMSNorm
-from .position import NoPositionEncoding, RotaryHalfSplit
+from .position import NoPositionEncoding, RotaryHalfSplit, RotaryInterleaved
+from .recurrent import MinGRU
 
 __all__ = [
-    "Block", "BuildContext", "CacheField", "CacheSpec", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
+    "Block", "BuildContext", "CacheField", "CacheSpec", "Carried", "LatentAttention", "MinGRU", "PostNormBlock",
+    "RoutedMLP", "RotaryInterleaved", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
     "NoPositionEncoding", "Norm", "NormFold", "Normed", "PagedAttention", "Part", "PartialSums", "PositionEncoding", "PreNormBlock", "Prenormed", "RMSNorm",
     "RotaryHalfSplit", "StateSpec",
 ]

@@ -143,6 +143,15 @@ class Normed:
 
 
 @dataclasses.dataclass
+class Carried:
+    """The rows of the residual stream in the activation type, with nothing left to add: what a
+    block that adds into the stream itself hands to the next one, which may read `x` instead
+    of converting the 32-bit rows once more."""
+
+    x: torch.Tensor  # [N, width], activation type (the stream itself where that is 32-bit)
+
+
+@dataclasses.dataclass
 class PartialSums:
     """A product that was taken in slices of its inner dimension and not added up yet:
     `sums` is float32 [slices, N, width], and the product is their sum in slice order.  Only a
@@ -175,6 +184,12 @@ class Norm(Part):
 
     def of_embedding(self, ids: torch.Tensor, table: torch.Tensor, step=None):
         return None
+
+    def add_normed(self, hidden: torch.Tensor, y: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """For arrangements that norm a sublayer's OUTPUT: hidden += norm(y [+ extra]) in 32-bit, in
+        place; returns the new rows of `hidden` in the activation type.  `y` and `extra` are
+        [N, width], each in the activation type or in 32-bit."""
+        raise NotImplementedError
 
     def fold(self, hidden: torch.Tensor) -> Optional[NormFold]:
         return None

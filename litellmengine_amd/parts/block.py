@@ -6,7 +6,9 @@ from __future__ import annotations
 from typing import Dict
 
 from ..weights.spec import TensorSpec
-from .base import Block, BuildContext, FeedForward, Mixer, Norm, Normed, Prenormed
+from typing import Optional
+
+from .base import Block, BuildContext, Carried, FeedForward, Mixer, Norm, Normed, Prenormed
 
 
 class PreNormBlock(Block):
@@ -37,6 +39,8 @@ class PreNormBlock(Block):
         return self.norm_in
 
     def forward(self, hidden, delta, step, cache, next_norm=None):
+        if isinstance(delta, Carried):  # the block before has added everything into the stream itself
+            delta = None
         if isinstance(delta, Prenormed):  # made for norm_in by the block before: the add and the norm are done
             x = delta
         elif isinstance(delta, Normed):  # norm_in's result, made together with the rows of `hidden`
@@ -52,3 +56,53 @@ class PreNormBlock(Block):
         if fold is not None:
             return self.feed_forward.forward(x, fold=fold)
         return self.feed_forward.forward(x)
+
+
+class PostNormBlock(Block):
+    """Residual block whose norms sit on the sublayers' OUTPUTS:
+        x <- x + norm_mix(mixer(x));  x <- x + norm_ff(ff(x))
+    The sublayers read the residual stream itself (its rows in the activation type).  Each
+    norm's kernel adds its result into the 32-bit stream and hands the new rows on in the
+    activation type, so a block leaves nothing to add: it returns a `Carried`.  A block
+    without a feed-forward is the first line alone."""
+
+    def __init__(self, norm_mix: Norm, mixer: Mixer, norm_ff: Optional[Norm] = None,
+                 feed_forward: Optional[FeedForward] = None):
+        if (norm_ff is None) != (feed_forward is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.norm_mix = norm_mix
+        self.mixer = mixer
+        self.norm_ff = norm_ff
+        self.feed_forward = feed_forward
+
+    def _parts(self):
+        return tuple(p for p in (self.norm_mix, self.mixer, self.norm_ff, self.feed_forward) if p is not None)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs: Dict[str, TensorSpec] = {}
+        for p in self._parts():
+            specs.update(p.tensor_specs())
+        return specs
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        for p in self._parts():
+            p.bind(weights, ctx)
+
+    def forward(self, hidden, delta, step, cache, next_norm=None):
+        if isinstance(delta, Carried):
+            x = delta.x
+        else:
+            if delta is not None:  # left by a block of another arrangement
+                if isinstance(delta, (Prenormed, Normed)):
+                    raise ValueError("a block that norms its sublayers' outputs takes no ready-made norm")
+                hidden += (delta.total() if hasattr(delta, "total") else delta).to(hidden.dtype)
+            x = self.ctx.ops.cast(hidden, self.ctx.dtype)
+        x = self.norm_mix.add_normed(hidden, self.mixer.forward(x, step, cache))
+        if self.feed_forward is not None:
+            y = self.feed_forward.forward(x)
+            extra = None
+            if isinstance(y, tuple):  # a feed-forward in two parts whose sum the norm's kernel takes
+                y, extra = y
+            x = self.norm_ff.add_normed(hidden, y, extra)
+        return Carried(x)

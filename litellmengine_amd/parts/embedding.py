@@ -11,7 +11,9 @@ from .base import BuildContext, Normed, Part
 
 
 class Embedding(Part):
-    def __init__(self, name: str, vocab_size: int, hidden_size: int):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, scale: float = 1.0):
+        """`scale`: every row is multiplied by it on its way into the 32-bit residual stream."""
+        self.scale = float(scale)
         self.name = name
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
@@ -29,6 +31,11 @@ class Embedding(Part):
         the tokens that the step before left on the device for their requests.  With `norm` (the
         parts.base.Norm that the first block begins with) the result is (rows, Normed or None):
         the norm's result comes along where one kernel makes both."""
+        if self.scale != 1.0:
+            feedback = step.token_feedback if step is not None else None
+            rows = self.ctx.ops.embedding(ids, self.weight, feedback, step.token_seq if feedback is not None else None,
+                                          step.seq_slots if feedback is not None else None, scale=self.scale)
+            return (rows, None) if norm is not None else rows
         if norm is not None:
             both = norm.of_embedding(ids, self.weight, step)
             if both is not None:

@@ -13,13 +13,16 @@ from .linear import Linear
 
 
 class GatedMLP(FeedForward):
-    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int):
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int,
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight"), to_residual: bool = True):
+        """`names`: the checkpoint's names of the gate, up and down weights after `prefix`.
+        `to_residual`: the result goes nowhere but into Norm.forward(hidden, delta) (it may then
+        come as PartialSums); an arrangement that does anything else with it says False."""
         # the products that do a folded norm's work read their inner dimension eight elements at a time
-        self.folds_norm = intermediate_size % 8 == 0
-        self.gate_up = Linear(
-            [prefix + "gate_proj.weight", prefix + "up_proj.weight"], hidden_size, [intermediate_size] * 2
-        )
-        self.down = Linear([prefix + "down_proj.weight"], intermediate_size, [hidden_size], to_residual=True)
+        self.folds_norm = intermediate_size % 8 == 0 and to_residual
+        gate, up, down = names
+        self.gate_up = Linear([prefix + gate, prefix + up], hidden_size, [intermediate_size] * 2)
+        self.down = Linear([prefix + down], intermediate_size, [hidden_size], to_residual=to_residual)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {**self.gate_up.tensor_specs(), **self.down.tensor_specs()}

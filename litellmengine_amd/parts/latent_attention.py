@@ -1,0 +1,98 @@
+"""Latent attention: keys and values of all heads are made from one small vector per token,
+and only that vector (and one rotated key part shared by the heads) is cached.
+
+    q = W_q h                          per head [dim plain | rot_dim rotated]
+    W_dkv h = [kv_rank | rot_dim]      c = RMSNorm(first part) * w   (the latent)
+                                       k_rot = rotated(second part)  (one for all heads)
+    per head: k_plain = W_uk c, v = W_uv c
+    score = (q_plain . k_plain + q_rot . k_rot) * scale
+    softmax over the keys AND one sink per head: the denominator also holds exp(sink_h)
+    out = W_o [heads' sum_j p_j v_j]
+
+Nothing per head is ever made for a cached token.  Since q_plain . (W_uk c) = (W_uk^T q_plain) . c
+and sum_j p_j (W_uv c_j) = W_uv (sum_j p_j c_j), a query is carried into the latent space once
+(`q_lat`, one small product per head), all heads of a token attend to the same cached rows
+[c | k_rot] as one multi-query attention whose values are the c rows themselves, and the
+result is expanded by W_uv once per query.  Prompt portions, decoded tokens and whole prompts
+are one case: the step's latents are written to their pages first, then every token attends
+through the block table.  Scores, softmax and sums are 32-bit in every mode.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Sequence
+
+import torch
+
+from ..weights.spec import INIT_NORM, INIT_NORMAL, TensorSpec
+from .base import BuildContext, CacheField, CacheSpec, Mixer
+from .linear import Linear
+from .position import RotaryInterleaved
+
+
+class LatentAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden_size: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
+                 scale: float, norm_eps: float, position: RotaryInterleaved, window: Optional[int] = None,
+                 names: Sequence[str] = ("q", "dkv", "dkv.norm", "uk", "uv", "sink", "o")):
+        """`position` rotates the first `position.rotary_dim` of the `rot_dim` elements.  `names`: the
+        checkpoint's names after `prefix` of the query projection, the down projection to
+        [latent | rotated key], the latent's norm weight, the up projections to plain keys and to
+        values, the sinks and the output projection."""
+        if position.rotary_dim > rot_dim:
+            raise ValueError("the rotation covers more elements than the rotated part has")
+        self.prefix = prefix
+        self.H, self.dim, self.rot, self.vdim, self.rank = heads, dim, rot_dim, vdim, kv_rank
+        self.scale = float(scale)
+        self.eps = float(norm_eps)
+        self.window = window
+        self.position = position
+        q, dkv, dkv_norm, uk, uv, sink, o = (prefix + n for n in names)
+        self.q = Linear([q], hidden_size, [heads * (dim + rot_dim)])
+        self.dkv = Linear([dkv], hidden_size, [kv_rank + rot_dim])
+        self.o = Linear([o], heads * vdim, [hidden_size])
+        self.norm_name, self.uk_name, self.uv_name, self.sink_name = dkv_norm, uk, uv, sink
+        self.norm_w = self.uk_t = self.uv = self.sink = None
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec((CacheField("c", 1, self.rank), CacheField("k_rot", 1, self.rot)), self.window)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {
+            **self.q.tensor_specs(), **self.dkv.tensor_specs(), **self.o.tensor_specs(),
+            self.norm_name: TensorSpec((self.rank,), INIT_NORM),
+            self.uk_name: TensorSpec((self.H * self.dim, self.rank), INIT_NORMAL),
+            self.uv_name: TensorSpec((self.H * self.vdim, self.rank), INIT_NORMAL),
+            self.sink_name: TensorSpec((self.H,), INIT_NORMAL),
+        }
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        for p in (self.q, self.dkv, self.o, self.position):
+            p.bind(weights, ctx)
+        self.norm_w = weights[self.norm_name].contiguous()
+        # per head, ready for `x . W^T`: W_uk^T [rank, dim] (queries into the latent space) and W_uv [vdim, rank]
+        uk = weights[self.uk_name].to(ctx.dtype).view(self.H, self.dim, self.rank)
+        self.uk_t = uk.transpose(1, 2).contiguous()
+        self.uv = weights[self.uv_name].to(ctx.dtype).view(self.H, self.vdim, self.rank).contiguous()
+        self.sink = weights[self.sink_name].float().contiguous()
+
+    def forward(self, x, step, cache):
+        ops = self.ctx.ops
+        group = cache.group
+        cos_sin = self.position.table(step)
+        rot_dims = self.position.rotary_dim
+        q = self.q.forward(x)
+        dkv = self.dkv.forward(x)
+        if cache.writes:
+            ops.latent_kv_write(dkv, self.norm_w, self.eps, cos_sin, rot_dims, group.slot_mapping, cache.pages,
+                                group.page_size, self.rank, self.rot)
+        q_rot = ops.latent_q_rope(q, cos_sin, rot_dims, self.H, self.dim, self.rot)
+        q_lat = ops.heads_linear(q, self.H, 0, self.dim, self.uk_t, torch.float32)  # [N, H, rank]
+        o_lat = ops.latent_attention(
+            q_lat, q_rot, cache.pages, group.page_size, self.rank, self.rot, group.block_table, step.seq_slots,
+            step.cu_tokens, step.kv_lens, step.token_seq, self.sink, self.window, self.scale, step.max_q_len,
+            step.max_kv_len, self.ctx.dtype,
+        )
+        v = ops.heads_linear(o_lat, self.H, 0, self.rank, self.uv, self.ctx.dtype)  # [N, H, vdim]
+        return self.o.forward(v.reshape(v.shape[0], self.H * self.vdim))

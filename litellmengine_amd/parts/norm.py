@@ -12,18 +12,25 @@ from .base import BuildContext, Norm, NormFold
 
 
 class RMSNorm(Norm):
-    def __init__(self, name: str, size: int, eps: float):
+    def __init__(self, name: str, size: int, eps: float, scalar: bool = False):
+        """`scalar`: the checkpoint holds ONE gain for all coordinates (a tensor without
+        dimensions); the kernels see it repeated `size` times."""
         self.name = name
         self.size = size
         self.eps = float(eps)
+        self.scalar = bool(scalar)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.name: TensorSpec((self.size,), INIT_NORM)}
+        return {self.name: TensorSpec(() if self.scalar else (self.size,), INIT_NORM)}
 
     def bind(self, weights, ctx: BuildContext) -> None:
         self.ctx = ctx
-        self.weight = weights[self.name].contiguous()  # bfloat16 or float32, as stored
+        w = weights[self.name]  # bfloat16 or float32, as stored
+        self.weight = (w.reshape(1).expand(self.size) if self.scalar else w).contiguous()
+
+    def add_normed(self, hidden, y, extra=None) -> torch.Tensor:
+        return self.ctx.ops.rmsnorm_add(hidden, y, self.weight, self.eps, self.ctx.dtype, extra)
 
     def forward(self, hidden, delta, rows=None) -> torch.Tensor:
         return self.ctx.ops.add_rmsnorm(hidden, delta, self.weight, self.eps, self.ctx.dtype, rows)

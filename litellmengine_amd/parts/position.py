@@ -48,3 +48,36 @@ class NoPositionEncoding(PositionEncoding):
 
     def fused_rotary(self, step):
         return None, 0
+
+
+class RotaryInterleaved(PositionEncoding):
+    """Rotary encoding with neighbouring pairs: element 2i pairs with 2i + 1 for i < dims / 2,
+    angle = pos * base^(-2i/dims),
+      y[2i] = x[2i] cos - x[2i+1] sin,  y[2i+1] = x[2i+1] cos + x[2i] sin;
+    elements from `dims` on pass unchanged.  The frequencies are computed once in double
+    precision and rounded to float32; angle, sine and cosine are float32, made once per step for
+    every layer with the same rotation (`table`), and applied by the mixer's own kernels."""
+
+    def __init__(self, dims: int, base: float):
+        if dims % 2 or dims < 0:
+            raise ValueError("a rotation takes an even number of elements")
+        self.rotary_dim = int(dims)
+        self.base = float(base)
+        self.inv_freq: Optional[torch.Tensor] = None
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+        inv = torch.pow(torch.tensor(self.base, dtype=torch.float64), -(2.0 * i) / max(1, self.rotary_dim))
+        self.inv_freq = inv.to(torch.float32).to(ctx.device)
+
+    def table(self, step) -> Optional[torch.Tensor]:
+        """float32 [N, dims / 2, 2] (cos, sin) of this step's positions; None without a rotation."""
+        if self.rotary_dim == 0:
+            return None
+        key = ("rope_table", self.base, self.rotary_dim)
+        table = step.scratch.get(key)
+        if table is None:
+            table = self.ctx.ops.rope_table(step.positions, self.inv_freq)
+            step.scratch[key] = table
+        return table

@@ -23,11 +23,11 @@ class TorchOps:
     def __init__(self, compute_dtype=torch.float64):
         self.cd = compute_dtype
 
-    def embedding(self, ids, table, feedback=None, token_seq=None, seq_slots=None):
+    def embedding(self, ids, table, feedback=None, token_seq=None, seq_slots=None, scale=1.0):
         ids = ids.long()
         if feedback is not None:
             ids = torch.where(ids < 0, feedback.long()[seq_slots.long()[token_seq.long()]], ids)
-        return table[ids].to(torch.float32)
+        return (table[ids].to(self.cd) * scale).to(torch.float32)
 
     def embedding_rmsnorm(self, ids, table, weight, eps, feedback=None, token_seq=None, seq_slots=None):
         hidden = self.embedding(ids, table, feedback, token_seq, seq_slots)
@@ -147,6 +147,125 @@ class TorchOps:
 
     def gate_up_silu(self, x, weight):
         return self.silu_mul(self.linear(x, weight))
+
+    # -- arrangements that norm a sublayer's output -------------------------------------------
+    def cast(self, x, dtype):
+        return x.to(dtype)
+
+    def scale_(self, x, factor):
+        x.copy_((x.to(self.cd) * factor).to(x.dtype))
+        return x
+
+    def rmsnorm_add(self, hidden, y, weight, eps, out_dtype, extra=None):
+        v = y.to(self.cd)
+        if extra is not None:
+            v = v + extra.to(self.cd)
+        v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight.to(self.cd)
+        hidden.copy_((hidden.to(self.cd) + v).to(hidden.dtype))
+        return hidden.to(out_dtype)
+
+    # -- gated recurrence --------------------------------------------------------------------
+    def mingru_scan(self, zxg, z_bias, x_bias, state, seq_slots, cu_tokens, out_dtype, max_q_len=0):
+        W = z_bias.shape[0]
+        v = zxg.to(self.cd)
+        z = torch.sigmoid(v[:, :W] + z_bias.to(self.cd))
+        u = v[:, W : 2 * W] + x_bias.to(self.cd)
+        c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+        g = v[:, 2 * W :]
+        g = g * torch.sigmoid(g)
+        out = torch.empty((zxg.shape[0], W), dtype=self.cd, device=zxg.device)
+        for s in range(seq_slots.shape[0]):
+            row = int(seq_slots[s])
+            S = state[row].to(self.cd)
+            for t in range(int(cu_tokens[s]), int(cu_tokens[s + 1])):
+                S = (1.0 - z[t]) * S + z[t] * c[t]
+                out[t] = S * g[t]
+            state[row] = S.to(state.dtype)
+        return out.to(out_dtype)
+
+    # -- latent attention --------------------------------------------------------------------
+    @staticmethod
+    def _rotate_pairs(x, cos_sin, rot_dims):
+        """x [N, ..., r]: pairs (2i, 2i + 1) of the first rot_dims elements turned by cos_sin [N, rot_dims / 2, 2]."""
+        if rot_dims == 0:
+            return x
+        y = x.clone()
+        shape = [x.shape[0]] + [1] * (x.dim() - 2) + [rot_dims // 2]
+        c, s = cos_sin[..., 0].to(x.dtype).view(shape), cos_sin[..., 1].to(x.dtype).view(shape)
+        u, v = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+        y[..., 0:rot_dims:2] = u * c - v * s
+        y[..., 1:rot_dims:2] = v * c + u * s
+        return y
+
+    def latent_kv_write(self, dkv, norm_w, eps, cos_sin, rot_dims, slots, pages, page_size, rank, rot):
+        x = dkv.to(self.cd)
+        c = x[:, :rank]
+        c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * norm_w.to(self.cd)
+        kr = self._rotate_pairs(x[:, rank:], cos_sin, rot_dims)
+        c_pages = pages[:, : page_size * rank].view(-1, page_size, rank)
+        r_pages = pages[:, page_size * rank : page_size * (rank + rot)].view(-1, page_size, rot)
+        for n in range(dkv.shape[0]):
+            slot = int(slots[n])
+            if slot < 0:
+                continue
+            c_pages[slot // page_size, slot % page_size] = c[n].to(pages.dtype)
+            r_pages[slot // page_size, slot % page_size] = kr[n].to(pages.dtype)
+
+    def latent_q_rope(self, q, cos_sin, rot_dims, heads, dim, rot):
+        x = q.view(q.shape[0], heads, dim + rot)[:, :, dim:].to(self.cd)
+        return self._rotate_pairs(x, cos_sin, rot_dims).to(torch.float32).contiguous()
+
+    def heads_linear(self, x, heads, col0, K, weight, out_dtype):
+        """x [N, heads * xw] or [N, heads, xw]; per head: columns col0 .. col0 + K of its part times weight[h] [out, K]^T."""
+        N = x.shape[0]
+        xs = x.reshape(N, heads, -1)[:, :, col0 : col0 + K].to(self.cd)
+        return torch.einsum("nhk,hok->nho", xs, weight.to(self.cd)).to(out_dtype).contiguous()
+
+    def latent_attention(self, q_lat, q_rot, pages, page_size, rank, rot, block_table, seq_slots, cu_tokens, kv_lens,
+                         token_seq, sink, window, scale, max_q_len, max_kv_len, out_dtype):
+        N, H, _ = q_lat.shape
+        c_pages = pages[:, : page_size * rank].view(-1, page_size, rank)
+        r_pages = pages[:, page_size * rank : page_size * (rank + rot)].view(-1, page_size, rot)
+        out = torch.zeros((N, H, rank), dtype=self.cd, device=pages.device)
+        for s in range(seq_slots.shape[0]):
+            row = int(seq_slots[s])
+            q0, q1 = int(cu_tokens[s]), int(cu_tokens[s + 1])
+            kv_len = int(kv_lens[s])
+            for t in range(q0, q1):
+                pos = kv_len - (q1 - q0) + (t - q0)
+                lo = max(0, pos - window + 1) if window else 0
+                idx = torch.arange(lo, pos + 1, device=pages.device)
+                pg = block_table[row, (idx // page_size).long()].long()
+                assert int(pg.min()) >= 0, "attention reads a page that was given back"
+                off = (idx % page_size).long()
+                c = c_pages[pg, off].to(self.cd)  # [n, rank]
+                kr = r_pages[pg, off].to(self.cd)
+                sc = (q_lat[t].to(self.cd) @ c.T + q_rot[t].to(self.cd) @ kr.T) * scale  # [H, n]
+                sk = sink.to(self.cd)[:, None]
+                m = torch.maximum(sc.max(dim=1, keepdim=True).values, sk)
+                e = torch.exp(sc - m)
+                out[t] = (e @ c) / (e.sum(1, keepdim=True) + torch.exp(sk - m))
+        return out.to(out_dtype)
+
+    # -- routed feed-forward -----------------------------------------------------------------
+    def moe_route(self, logits, bias, top):
+        v = logits.to(self.cd) + bias.to(self.cd)
+        vals, idx = torch.topk(v, top, dim=-1)
+        return idx.to(torch.int32), torch.softmax(vals, dim=-1).to(torch.float32)
+
+    def moe_experts(self, x, ids, gains, gate_up, down):
+        N, top = ids.shape
+        ff = gate_up.shape[1] // 2
+        out = torch.zeros((N, down.shape[1]), dtype=self.cd, device=x.device)
+        xx = x.to(self.cd)
+        for n in range(N):
+            for k in range(top):
+                e = int(ids[n, k])
+                gu = gate_up[e].to(self.cd) @ xx[n]
+                a = gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]
+                a = a.to(x.dtype).to(self.cd)
+                out[n] += gains[n, k].to(self.cd) * (down[e].to(self.cd) @ a)
+        return out.to(torch.float32)
 
     def argmax(self, logits, scatter=None):
         out = torch.argmax(logits, dim=-1).to(torch.int32)  # torch returns the first maximum
