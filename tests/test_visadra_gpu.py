@@ -1,0 +1,160 @@
+"""Visadra on the GPU: bin/trace_run as a child process (whole prompts, decoded tails, portions
+down to two tokens, mixed batches in a pool of the live peak with four slots) in float32 and
+bfloat16 against the plain model, with random weights and with weights made so that single keys,
+the sink, the recurrences' memory and the routers' choices carry the result; long decoding across
+windows; generation through the Python entry point and the command line."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests.plain import visadra_plain as plain
+from tests.tiny import random_tokens
+from tests.trace_util import ROOT, TraceBuilder, changing_portions, check_dumps, mixed, tail_one_by_one, whole
+from tests.visadra_util import CONFIGS, PAGE_SIZES, attention_peaks, make_model_dir, plain_logits, run_tool, sharpen
+
+pytestmark = pytest.mark.gpu
+
+# about five times the worst error seen (float32 1e-6, bfloat16 6e-3 at these sizes)
+TOL = {"float32": 1e-5, "bfloat16": 3e-2}
+LENGTHS = {"a": 70, "b": 45, "c": 100, "d": 33, "e": 64, "f": 1, "g": 2}
+
+
+def all_ways_trace(requests, tail=32):
+    tb = TraceBuilder()
+    names = list(requests)
+    whole(tb, names[0] + "#whole", requests[names[0]])
+    whole(tb, names[2] + "#whole", requests[names[2]])
+    tail_one_by_one(tb, names[1] + "#tail", requests[names[1]], tail=tail)
+    changing_portions(tb, names[2] + "#cut", requests[names[2]], seed=1)
+    changing_portions(tb, names[4] + "#cut", requests[names[4]], seed=2)
+    mixed(tb, {rid + "#mix": t for rid, t in requests.items()}, seed=5)
+    return tb
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "A/default page", "B", "C"])
+def test_trace_gpu(tmp_path, which, dtype):
+    which, default_page = which[0], len(which) > 1
+    d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
+    sharpen(d, fixed_routes=dtype == "bfloat16")
+    vocab = CONFIGS[which]["vocab"]
+    requests = {rid: random_tokens(n, vocab, 10 + i) for i, (rid, n) in enumerate(LENGTHS.items())}
+    tb = all_ways_trace(requests)
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=None if default_page else PAGE_SIZES[which])
+    worst = check_dumps(out, tb, plain_logits(d, requests), TOL[dtype])
+    print(f"trace {which} {dtype}: worst relative error {worst:.3g}, pool {tb.max_tokens} tokens")
+
+
+# Larger scores carry the rounding of queries and latents further into the softmax weights, and
+# sharper gates carry the rounding of their inputs into the states: the tolerances grow with the factors.
+# (B's scores grow faster with the factor: more elements per head and a larger scale)
+PEAK = {("A", "float32"): (17.0, 20.0, 1e-4), ("A", "bfloat16"): (12.0, 10.0, 1e-1),
+        ("B", "float32"): (10.0, 10.0, 1e-4), ("B", "bfloat16"): (5.0, 5.0, 1e-1)}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_trace_with_single_keys_standing_out(tmp_path, which, dtype):
+    """Requests of hundreds of tokens whose attention picks out single keys, near, far back and at the
+    windows' edges (19 and 48 keys), whose first head's sink takes a real share, whose recurrences
+    remember or forget sharply and whose routers choose clearly; the last 80 tokens of one request are
+    decoded one by one, so the windows pass over decoded tokens."""
+    d = make_model_dir(tmp_path, which, seed=5, dtype=torch.bfloat16)
+    factor, gates, tol = PEAK[which, dtype]
+    sharpen(d, factor, sink=2.0, gates=gates, fixed_routes=dtype == "bfloat16")
+    vocab = CONFIGS[which]["vocab"]
+    requests = {"p": random_tokens(300, vocab, 41), "q": random_tokens(170, vocab, 42),
+                "r": random_tokens(230, vocab, 43), "s": random_tokens(90, vocab, 44)}
+    assert attention_peaks(d, requests["q"]) > 0.15
+    tb = TraceBuilder()
+    whole(tb, "p#whole", requests["p"])
+    tail_one_by_one(tb, "p#tail", requests["p"], tail=80)
+    changing_portions(tb, "r#cut", requests["r"], seed=3)
+    mixed(tb, {rid + "#mix": t for rid, t in requests.items()}, seed=6)
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=PAGE_SIZES[which])
+    worst = check_dumps(out, tb, plain_logits(d, requests), tol)
+    print(f"peaked trace {which} {dtype}: worst relative error {worst:.3g}")
+
+
+def test_a_lost_key_or_a_lost_sink_would_show(tmp_path):
+    """The measure of the test above: in the plain model of its weights, dropping the key at a window's far
+    edge, or the sink, moves the logits of most positions by more than ten times the 32-bit tolerance
+    (and of some by a third of the largest logit)."""
+    d = make_model_dir(tmp_path, "A", seed=5, dtype=torch.bfloat16)
+    sharpen(d, 12.0, sink=2.0, gates=10.0, fixed_routes=True)
+    cfg, w = plain.read_model_dir(d)
+    tokens = random_tokens(120, cfg["vocab"], 42)
+    base = plain.model_logits(tokens, w, cfg)
+    narrower = {**cfg, "layers": [dict(l, mixer=dict(l["mixer"], window=l["mixer"]["window"] - 1))
+                                  if l["mixer"].get("window") else l for l in cfg["layers"]]}
+    moved = (plain.model_logits(tokens, w, narrower) - base).abs().max(dim=1).values / base.abs().max()
+    assert float((moved[30:] > 1e-3).float().mean()) > 0.5 and float(moved.max()) > 0.1
+    no_sink = {k: (v - 100.0 if k.endswith(".sink") else v) for k, v in w.items()}
+    moved = (plain.model_logits(tokens, no_sink, cfg) - base).abs().max(dim=1).values / base.abs().max()
+    assert float((moved > 1e-3).float().mean()) > 0.5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_in_a_batch_with_slots_used_again(tmp_path, dtype):
+    """Three requests decode 150 tokens each side by side (captured graphs), the shortest ends and its
+    slot and pages go to a newcomer whose prompt runs beside the others' single tokens."""
+    d = make_model_dir(tmp_path, "B", seed=9, dtype=torch.bfloat16)
+    sharpen(d, 8.0 if dtype == "float32" else 4.0, gates=5.0, fixed_routes=dtype == "bfloat16")
+    vocab = CONFIGS["B"]["vocab"]
+    requests = {rid: random_tokens(n, vocab, 60 + i) for i, (rid, n) in enumerate({"a": 170, "b": 200, "c": 230, "n": 90}.items())}
+    tb = TraceBuilder()
+    tb.step([(r, requests[r][: len(requests[r]) - 150], [0]) for r in "abc"])
+    live, at = ["a", "b", "c"], {r: len(requests[r]) - 150 for r in "abc"}
+    at["n"] = 0
+    for i in range(150):
+        entries, end = [], []
+        for r in list(live):
+            n = 40 if r == "n" and at[r] == 0 else 1
+            entries.append((r, requests[r][at[r] : at[r] + n], [n - 1]))
+            at[r] += n
+            if at[r] == len(requests[r]):
+                end.append(r)
+                live.remove(r)
+        tb.step(entries, end)
+        if i == 20:
+            live.remove("a")
+            tb.steps[-1]["end"].append("a")
+            tb.live.pop("a")
+            live.append("n")
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=16, max_requests=3)
+    worst = check_dumps(out, tb, plain_logits(d, requests), 1e-4 if dtype == "float32" else 1e-1)
+    print(f"long decoding {dtype}: worst relative error {worst:.3g}")
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(tmp_path, which):
+    from litellmengine_amd.entrypoints.generate import generate
+
+    d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
+    cfg, w = plain.read_model_dir(d)
+    prompts = [random_tokens(n, cfg["vocab"], 70 + i) for i, n in enumerate((1, 7, 23, 60))]
+    want = [plain.generate_greedy(p, w, cfg, 12) for p in prompts]
+    assert generate(d, prompts, max_tokens=12, dtype="float32", page_size=PAGE_SIZES[which]) == want
+    # portions, and a pool in which requests are preempted and recomputed
+    assert generate(d, prompts, max_tokens=12, dtype="float32", page_size=8, prefill_chunk=16,
+                    max_tokens_per_step=24, num_pages=14) == want
+
+
+def test_command_line_generates(tmp_path):
+    d = make_model_dir(tmp_path, "B", dtype=torch.bfloat16)
+    cfg, w = plain.read_model_dir(d)
+    prompt = random_tokens(19, cfg["vocab"], 80)
+    want = plain.generate_greedy(prompt, w, cfg, 10)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "litellmengine"), "--model", d, "--input-ids",
+                           ",".join(map(str, prompt)), "--max-tokens", "10", "--temperature", "0", "--dtype", "float32"],
+                          text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.split("\n")
+    got = [int(t) for t in lines[lines.index("New token ids:") + 1].replace(" ", "").split(",")]
+    assert got == want
