@@ -1,6 +1,7 @@
 // Latent attention: the cache holds, per token, one latent row c [rank] and one rotated key part
-// k_rot [rot] shared by all heads; a page is [page_size][rank] of c followed by
-// [page_size][rot] of k_rot.  Queries arrive already carried into the latent space
+// k_rot [rot] shared by all heads; a page is [page_size][rank] of c, then the same latents
+// transposed, [rank][page_size] (the matrix cores contract over keys in the second product and
+// want the keys of one element side by side), then [page_size][rot] of k_rot.  Queries arrive already carried into the latent space
 // (q_lat [N, H, rank], float32 or the cache's type) together with their rotated part
 // (q_rot [N, H, rot], float32), so all heads of a token attend to the same rows:
 //   score_j = (q_lat . c_j + q_rot . k_rot_j) * scale
@@ -36,9 +37,13 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restric
     const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
     T* page = pages + (int64_t)(slot / P) * page_stride;
     T* c = page + (int64_t)(slot % P) * rank;
-    T* kr = page + (int64_t)P * rank + (int64_t)(slot % P) * rot;
-    for (int i = threadIdx.x; i < rank; i += blockDim.x)
-        c[i] = from_f32<T>(to_f32<T>(row[i]) * inv * load_as_f32(norm_w, i, w_dtype));
+    T* ct = page + (int64_t)P * rank + (slot % P);
+    T* kr = page + (int64_t)2 * P * rank + (int64_t)(slot % P) * rot;
+    for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+        const T v = from_f32<T>(to_f32<T>(row[i]) * inv * load_as_f32(norm_w, i, w_dtype));
+        c[i] = v;
+        ct[(int64_t)i * P] = v;
+    }
     const float* cs = cos_sin + n * rot_dims;  // [rot_dims / 2][2]
     for (int i = threadIdx.x; i < rot; i += blockDim.x) {
         float v = to_f32<T>(row[rank + i]);
@@ -157,7 +162,7 @@ __global__ __launch_bounds__(LAT_TILE) void latent_attention_generic_kernel(
             const T* pg = pages + (int64_t)page * page_stride;
             const int64_t c_at = (int64_t)(j % P) * rank;
             const T* c = pg + c_at;
-            const T* kr = pg + (int64_t)P * rank + (int64_t)(j % P) * rot;
+            const T* kr = pg + (int64_t)2 * P * rank + (int64_t)(j % P) * rot;
             float dot = 0.f;
             for (int i = 0; i < rank; ++i) dot += qa[i] * to_f32<T>(c[i]);
             for (int i = 0; i < rot; ++i) dot += qr[i] * to_f32<T>(kr[i]);
@@ -214,5 +219,237 @@ extern "C" int lle_latent_attention_generic(const void* q_lat, int q_lat_dtype, 
     else
         latent_attention_generic_kernel<bf16_t, bf16_t><<<grid, LAT_TILE, lds, stream>>>(LAT_ARGS(bf16_t, bf16_t));
 #undef LAT_ARGS
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// bfloat16 on the matrix cores.  The rows of a request are its (token, head) pairs, token after
+// token; a wavefront takes one tile of 16 rows over a range of 32-key steps:
+//   S^T = K Q^T      A = [16 keys x 32 elements] of [c | k_rot], B = the queries (in registers)
+//   O^T += C^T P^T   A = [16 latent elements x 32 keys] of the transposed latents, B = P^T
+// With v_mfma_f32_16x16x32_bf16 lane (c = lane / 16, r = lane % 16) holds of a result tile column r,
+// rows 4c .. 4c + 3.  Row q of K tile x stands for key 8 (q / 4) + 4 x + q % 4 of the step, so the
+// lane's eight scores are the consecutive keys 8c .. 8c + 7 of query row r: the B operand of the
+// second product as it stands, and its A operand is one 16-byte piece of the transposed page.
+// The softmax state of row r lives in the four lanes r + 16c.  Every operand comes straight from
+// the pages (no LDS: wavefronts are independent, one per workgroup).  With `nsplit` > 1 a tile's
+// keys are cut into ranges whose unnormalised results (and m, l) go to a workspace and are merged
+// by latent_combine_kernel; the sink (m = sink, l = 1) belongs to the first range.
+// RK = 32-element steps over the latent (rank <= 32 RK, padded with zeros), RR the same for k_rot.
+// ---------------------------------------------------------------------------------------------
+typedef bf16_t lbf16x8 __attribute__((ext_vector_type(8)));
+typedef bf16_t lbf16x4 __attribute__((ext_vector_type(4)));
+typedef float lf32x4 __attribute__((ext_vector_type(4)));
+#define LAT_NEG_BIG (-1.0e30f)
+#define LAT_LOG2E 1.4426950408889634f
+
+__device__ __forceinline__ lbf16x8 lat_zero8() {
+    lbf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (bf16_t)0.0f;
+    return z;
+}
+
+template <int RK, int RR>
+__global__ __launch_bounds__(64) void latent_attention_mfma_kernel(
+    const bf16_t* __restrict__ q_lat, int64_t ql_stride_n, int64_t ql_stride_h, const float* __restrict__ q_rot,
+    const bf16_t* __restrict__ pages, int64_t page_stride, int P, int rank, int rot,
+    const int32_t* __restrict__ block_table, int max_pages, const int32_t* __restrict__ seq_slots,
+    const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ kv_lens, const float* __restrict__ sink,
+    int window, float scale, bf16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml, int H,
+    int tiles_max, int nsplit) {
+    const int lane = threadIdx.x, c = lane / 16, r = lane % 16;
+    int item = blockIdx.x;
+    const int split = item % nsplit;
+    item /= nsplit;
+    const int tile = item % tiles_max, s = item / tiles_max;
+    const int q0 = cu_tokens[s], q_len = cu_tokens[s + 1] - q0;
+    const int rows = q_len * H;
+    if (tile * 16 >= rows) return;  // (the whole wavefront)
+    const int past = kv_lens[s] - q_len;
+    const int rho = tile * 16 + r;
+    const bool valid = rho < rows;
+    const int t = valid ? rho / H : 0, h = valid ? rho % H : 0;
+    const int pos = valid ? past + t : -1;  // a row that does not exist sees nothing
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int t_first = (tile * 16) / H, t_last = min(q_len - 1, (tile * 16 + 15) / H);
+    const int kmax = past + t_last;  // the tile's keys: lo_min .. kmax
+    const int lo_min = window > 0 ? max(0, past + t_first - window + 1) : 0;
+    const int32_t* table = block_table + (int64_t)seq_slots[s] * max_pages;
+
+    lbf16x8 qv[RK + RR];
+    {
+        const bf16_t* ql = q_lat + (int64_t)(q0 + t) * ql_stride_n + (int64_t)h * ql_stride_h;
+#pragma unroll
+        for (int ks = 0; ks < RK; ++ks) {
+            const int e0 = 32 * ks + 8 * c;
+            qv[ks] = (valid && e0 < rank) ? *(const lbf16x8*)(ql + e0) : lat_zero8();
+        }
+        const float* qr = q_rot + ((int64_t)(q0 + t) * H + h) * rot;
+#pragma unroll
+        for (int kr = 0; kr < RR; ++kr) {
+            const int e0 = 32 * kr + 8 * c;
+            lbf16x8 v = lat_zero8();
+            if (valid && e0 < rot) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = (bf16_t)qr[e0 + i];
+            }
+            qv[RK + kr] = v;
+        }
+    }
+    lf32x4 o[2 * RK];
+#pragma unroll
+    for (int n = 0; n < 2 * RK; ++n) o[n] = lf32x4{0.f, 0.f, 0.f, 0.f};
+    const bool first = split == 0 && valid;
+    float m = first ? sink[h] * LAT_LOG2E : LAT_NEG_BIG;  // base 2
+    float l = (first && c == 0) ? 1.0f : 0.0f;            // this lane's share of the row's sum
+    const float sc2 = scale * LAT_LOG2E;
+
+    const int s_begin = lo_min / 32, s_end = kmax / 32 + 1;
+    const int per = (s_end - s_begin + nsplit - 1) / nsplit;
+    const int st_lo = s_begin + split * per, st_hi = min(s_end, st_lo + per);
+    for (int st = st_lo; st < st_hi; ++st) {
+        const int j0 = st * 32;
+        lf32x4 sacc[2];
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            sacc[x] = lf32x4{0.f, 0.f, 0.f, 0.f};
+            const int key = j0 + 8 * (r / 4) + 4 * x + r % 4;
+            const bool ok = key >= lo_min && key <= kmax;
+            const bf16_t* pg = pages + (int64_t)(ok ? table[key / P] : 0) * page_stride;
+            const bf16_t* kp = pg + (int64_t)(key % P) * rank;
+            const bf16_t* krp = pg + (int64_t)2 * P * rank + (int64_t)(key % P) * rot;
+#pragma unroll
+            for (int ks = 0; ks < RK; ++ks) {
+                const int e0 = 32 * ks + 8 * c;
+                const lbf16x8 a = (ok && e0 < rank) ? *(const lbf16x8*)(kp + e0) : lat_zero8();
+                sacc[x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qv[ks], sacc[x], 0, 0, 0);
+            }
+#pragma unroll
+            for (int kr = 0; kr < RR; ++kr) {
+                const int e0 = 32 * kr + 8 * c;
+                const lbf16x8 a = (ok && e0 < rot) ? *(const lbf16x8*)(krp + e0) : lat_zero8();
+                sacc[x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qv[RK + kr], sacc[x], 0, 0, 0);
+            }
+        }
+        float sv[8];
+        float mx = LAT_NEG_BIG;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int key = j0 + 8 * c + i;
+            const float v = (i < 4 ? sacc[0][i] : sacc[1][i - 4]) * sc2;
+            sv[i] = (key >= lo && key <= pos) ? v : LAT_NEG_BIG;
+            mx = fmaxf(mx, sv[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, LLE_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, LLE_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float alpha = exp2f(m - m_new);
+        lbf16x8 pb;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float p = sv[i] <= 0.5f * LAT_NEG_BIG ? 0.f : exp2f(sv[i] - m_new);
+            psum += p;
+            pb[i] = (bf16_t)p;
+        }
+        l = l * alpha + psum;
+        m = m_new;
+        const int gkey = j0 + 8 * c;  // this lane's eight keys, inside one page
+        const bool gok = gkey + 7 >= lo_min && gkey <= kmax;
+        const bf16_t* vt = pages + (int64_t)(gok ? table[gkey / P] : 0) * page_stride + (int64_t)P * rank + gkey % P;
+#pragma unroll
+        for (int n = 0; n < 2 * RK; ++n) {
+            if (16 * n < rank) {
+                o[n] *= alpha;
+                const lbf16x8 a = gok ? *(const lbf16x8*)(vt + (int64_t)(16 * n + r) * P) : lat_zero8();
+                o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[n], 0, 0, 0);
+            }
+        }
+    }
+    l += __shfl_xor(l, 16, LLE_WAVE);
+    l += __shfl_xor(l, 32, LLE_WAVE);
+    if (!valid) return;
+    const int64_t grow = (int64_t)(q0 + t) * H + h;
+    if (nsplit == 1) {
+        const float inv = 1.0f / l;
+        bf16_t* orow = out + grow * rank;
+#pragma unroll
+        for (int n = 0; n < 2 * RK; ++n) {
+            if (16 * n < rank) {
+                lbf16x4 v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(o[n][i] * inv);
+                *(lbf16x4*)(orow + 16 * n + 4 * c) = v;
+            }
+        }
+    } else {
+        float* wo = ws_o + (grow * nsplit + split) * rank;
+#pragma unroll
+        for (int n = 0; n < 2 * RK; ++n)
+            if (16 * n < rank) *(lf32x4*)(wo + 16 * n + 4 * c) = o[n];
+        if (c == 0) {
+            ws_ml[(grow * nsplit + split) * 2] = m;
+            ws_ml[(grow * nsplit + split) * 2 + 1] = l;
+        }
+    }
+}
+
+// one workgroup per (token, head): the ranges' results weighted by 2^(m_i - max m) and normalised
+__global__ __launch_bounds__(128) void latent_combine_kernel(const float* __restrict__ ws_o,
+                                                              const float* __restrict__ ws_ml,
+                                                              bf16_t* __restrict__ out, int rank, int nsplit) {
+    const int64_t row = blockIdx.x;
+    const float* ml = ws_ml + row * nsplit * 2;
+    float M = LAT_NEG_BIG;
+    for (int i = 0; i < nsplit; ++i) M = fmaxf(M, ml[2 * i]);
+    float L = 0.f;
+    for (int i = 0; i < nsplit; ++i) L += ml[2 * i + 1] * exp2f(ml[2 * i] - M);
+    const float inv = 1.0f / L;
+    for (int e = threadIdx.x; e < rank; e += blockDim.x) {
+        float acc = 0.f;
+        for (int i = 0; i < nsplit; ++i) acc += ws_o[(row * nsplit + i) * rank + e] * exp2f(ml[2 * i] - M);
+        out[row * rank + e] = (bf16_t)(acc * inv);
+    }
+}
+
+// q_lat bfloat16 [N, H, rank] with strides that are multiples of 8; rank a multiple of 16 up to 512, rot a
+// multiple of 8 up to 64, P a multiple of 16.  `tiles_max` = ceil(max_q_len * H / 16).  nsplit > 1 needs
+// ws_o float32 [N H nsplit rank] and ws_ml float32 [N H nsplit 2].
+extern "C" int lle_latent_attention_mfma(const void* q_lat, int64_t ql_stride_n, int64_t ql_stride_h,
+                                         const void* q_rot, const void* pages, int64_t page_stride, int P, int rank,
+                                         int rot, const void* block_table, int max_pages, const void* seq_slots,
+                                         const void* cu_tokens, const void* kv_lens, const void* sink, int window,
+                                         float scale, void* out, void* ws_o, void* ws_ml, int N, int S, int H,
+                                         int tiles_max, int nsplit, hipStream_t stream) {
+    if (N <= 0 || S <= 0 || H <= 0 || tiles_max <= 0) return 0;
+    if (rank <= 0 || rank > 512 || rank % 16 || rot < 0 || rot > 64 || rot % 8 || P <= 0 || P % 16 ||
+        ql_stride_n % 8 || ql_stride_h % 8 || page_stride % 8 || nsplit < 1 || (nsplit > 1 && (!ws_o || !ws_ml)))
+        return (int)hipErrorInvalidValue;
+    const int64_t items = (int64_t)S * tiles_max * nsplit;
+    if (items > 0x7fffffff) return (int)hipErrorInvalidValue;
+    const int RK = rank <= 64 ? 2 : rank <= 128 ? 4 : rank <= 256 ? 8 : 16;
+    const int RR = rot <= 32 ? 1 : 2;
+#define LAT_LAUNCH(K, R)                                                                                              \
+    latent_attention_mfma_kernel<K, R><<<(int)items, 64, 0, stream>>>(                                                \
+        (const bf16_t*)q_lat, ql_stride_n, ql_stride_h, (const float*)q_rot, (const bf16_t*)pages, page_stride, P,    \
+        rank, rot, (const int32_t*)block_table, max_pages, (const int32_t*)seq_slots, (const int32_t*)cu_tokens,      \
+        (const int32_t*)kv_lens, (const float*)sink, window, scale, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, H,     \
+        tiles_max, nsplit)
+    if (RR == 1) {
+        if (RK == 2) LAT_LAUNCH(2, 1);
+        else if (RK == 4) LAT_LAUNCH(4, 1);
+        else if (RK == 8) LAT_LAUNCH(8, 1);
+        else LAT_LAUNCH(16, 1);
+    } else {
+        if (RK == 2) LAT_LAUNCH(2, 2);
+        else if (RK == 4) LAT_LAUNCH(4, 2);
+        else if (RK == 8) LAT_LAUNCH(8, 2);
+        else LAT_LAUNCH(16, 2);
+    }
+#undef LAT_LAUNCH
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    if (nsplit > 1) latent_combine_kernel<<<N * H, 128, 0, stream>>>((const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, rank, nsplit);
     LLE_RETURN_LAUNCH_STATUS();
 }

@@ -747,14 +747,15 @@ class HipOps:
                         rank: int, rot: int) -> None:
         """dkv [N, rank + rot] -> the pages: c = RMSNorm(first rank) * norm_w and the rest with its first
         `rot_dims` elements rotated in neighbouring pairs by cos_sin [N, rot_dims / 2, 2].  A page
-        (one row of `pages`) is [page_size][rank] then [page_size][rot]; slots[n] < 0 writes nothing."""
+        (one row of `pages`) is the latents [page_size][rank], the same transposed [rank][page_size],
+        then the rotated parts [page_size][rot]; slots[n] < 0 writes nothing."""
         _dev(dkv, "dkv")
         _dev(norm_w, "latent norm weight")
         _dev(slots, "slots", torch.int32)
         N = dkv.shape[0]
         _need(dkv.shape == (N, rank + rot) and norm_w.shape == (rank,) and slots.shape == (N,), "dkv [N, rank + rot]")
         _need(pages.is_cuda and pages.dtype == dkv.dtype and pages.dim() == 2 and pages.stride(1) == 1
-              and pages.shape[1] >= page_size * (rank + rot), "pages must be [pages, page_size * (rank + rot)]")
+              and pages.shape[1] >= page_size * (2 * rank + rot), "pages must be [pages, page_size * (2 rank + rot)]")
         if rot_dims:
             _dev(cos_sin, "cos_sin", torch.float32)
             _need(cos_sin.shape == (N, rot_dims // 2, 2), "cos_sin must be [N, rot_dims / 2, 2]")
@@ -807,6 +808,25 @@ class HipOps:
                           a_ptr, b_ptr, c_ptr, N, O, K, heads * xw, K, heads * O, F32, F32)
         return out
 
+    force_generic_latent = False  # tests flip this to compare the two kernels
+    last_latent_kernel = None  # (which kernel, key ranges) of the last latent_attention call: for tests
+
+    def latent_query_dtype(self, cache_dtype, page_size: int, rank: int, rot: int):
+        """The type in which latent_attention wants q_lat: the cache's where the matrix-core kernel takes the
+        sizes (bfloat16, rank a multiple of 16 up to 512, rot a multiple of 8 up to 64, pages of a multiple of
+        16 tokens), float32 otherwise."""
+        mfma = (cache_dtype == torch.bfloat16 and rank % 16 == 0 and rank <= 512 and rot % 8 == 0 and rot <= 64
+                and page_size % 16 == 0 and not self.force_generic_latent)
+        return torch.bfloat16 if mfma else torch.float32
+
+    def latent_splits(self, num_seqs: int, heads: int, max_q_len: int, max_kv_len: int, window: int) -> int:
+        """Key ranges per 16-row tile of the matrix-core kernel: enough wavefronts for four on every CU,
+        at least two 32-key steps each, at most 64."""
+        tiles = max(1, num_seqs) * -(-max(1, max_q_len) * heads // 16)
+        span = min(max_kv_len, window + max_q_len) if window else max_kv_len
+        steps = -(-max(1, span) // 32)
+        return int(max(1, min(-(-4 * self.compute_units() // tiles), steps // 2, 64)))
+
     def latent_attention(self, q_lat, q_rot, pages, page_size: int, rank: int, rot: int, block_table, seq_slots,
                          cu_tokens, kv_lens, token_seq, sink, window: Optional[int], scale: float, max_q_len: int,
                          max_kv_len: int, out_dtype) -> torch.Tensor:
@@ -825,11 +845,30 @@ class HipOps:
         _need(q_lat.dtype in (torch.float32, pages.dtype), "q_lat is float32 or of the cache's type")
         _need(q_rot.shape == (N, H, rot) and sink.shape == (H,), "q_rot [N, H, rot], sink [H]")
         _need(pages.is_cuda and pages.dim() == 2 and pages.stride(1) == 1 and pages.dtype == out_dtype
-              and pages.shape[1] >= page_size * (rank + rot), "pages must be [pages, page_size * (rank + rot)]")
+              and pages.shape[1] >= page_size * (2 * rank + rot), "pages must be [pages, page_size * (2 rank + rot)]")
         _need(token_seq.shape == (N,) and cu_tokens.shape == (S + 1,) and kv_lens.shape == (S,), "the step's arrays")
         _need(block_table.dim() == 2, "block_table must be [slots, pages]")
         _need(rank <= 1024, f"a latent of {rank} elements is wider than the attention kernels take (1024)")
         out = torch.empty((N, H, rank), dtype=out_dtype, device=pages.device)
+        win = int(window) if window else 0
+        if (q_lat.dtype == torch.bfloat16 and self.latent_query_dtype(pages.dtype, page_size, rank, rot) == torch.bfloat16
+                and q_lat.stride(0) % 8 == 0 and q_lat.stride(1) % 8 == 0 and pages.stride(0) % 8 == 0
+                and max_q_len > 0 and max_kv_len > 0):
+            ns = self.latent_splits(S, H, max_q_len, max_kv_len, win)
+            self.last_latent_kernel = ("matrix cores", ns)
+            ws_o = ws_ml = None
+            if ns > 1:
+                ws_o = torch.empty((N * H * ns * rank,), dtype=torch.float32, device=pages.device)
+                ws_ml = torch.empty((N * H * ns * 2,), dtype=torch.float32, device=pages.device)
+            self._run("latent", "lle_latent_attention_mfma",
+                      [_P, _L, _L, _P, _P, _L, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _F, _P, _P, _P, _I, _I, _I, _I, _I,
+                       _P],
+                      _ptr(q_lat), q_lat.stride(0), q_lat.stride(1), _ptr(q_rot), _ptr(pages), pages.stride(0),
+                      int(page_size), rank, rot, _ptr(block_table), block_table.shape[1], _ptr(seq_slots),
+                      _ptr(cu_tokens), _ptr(kv_lens), _ptr(sink), win, float(scale), _ptr(out), _ptr(ws_o), _ptr(ws_ml),
+                      N, S, H, -(-max_q_len * H // 16), ns)
+            return out
+        self.last_latent_kernel = ("generic", 1)
         self._run("latent", "lle_latent_attention_generic",
                   [_P, _I, _L, _L, _P, _P, _L, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _F, _P, _I, _I, _I, _P],
                   _ptr(q_lat), dtype_code(q_lat.dtype), q_lat.stride(0), q_lat.stride(1), _ptr(q_rot), _ptr(pages),

@@ -55,7 +55,10 @@ class LatentAttention(Mixer):
         self.norm_w = self.uk_t = self.uv = self.sink = None
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec((CacheField("c", 1, self.rank), CacheField("k_rot", 1, self.rot)), self.window)
+        # the latents twice: token after token for the scores, transposed (the keys of one element
+        # side by side) for the weighted sum, which the matrix cores contract over keys
+        return CacheSpec((CacheField("c", 1, self.rank), CacheField("c_t", 1, self.rank, True),
+                          CacheField("k_rot", 1, self.rot)), self.window)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {
@@ -88,7 +91,8 @@ class LatentAttention(Mixer):
             ops.latent_kv_write(dkv, self.norm_w, self.eps, cos_sin, rot_dims, group.slot_mapping, cache.pages,
                                 group.page_size, self.rank, self.rot)
         q_rot = ops.latent_q_rope(q, cos_sin, rot_dims, self.H, self.dim, self.rot)
-        q_lat = ops.heads_linear(q, self.H, 0, self.dim, self.uk_t, torch.float32)  # [N, H, rank]
+        q_lat = ops.heads_linear(q, self.H, 0, self.dim, self.uk_t,
+                                 ops.latent_query_dtype(self.ctx.dtype, group.page_size, self.rank, self.rot))  # [N, H, rank]
         o_lat = ops.latent_attention(
             q_lat, q_rot, cache.pages, group.page_size, self.rank, self.rot, group.block_table, step.seq_slots,
             step.cu_tokens, step.kv_lens, step.token_seq, self.sink, self.window, self.scale, step.max_q_len,

@@ -99,7 +99,9 @@ def latent_case(dtype, P, rank, rot, H, lens, pasts, seed, pages_total=64):
             slot_map.append(int(table[slots_of[s], t // P]) * P + t % P)
             token_seq.append(s)
         cu.append(cu[-1] + n)
-    pages = rnd((pages_total + 1, P * (rank + rot) + 3), dtype, seed + 1)[:, : P * (rank + rot)]  # rows with a stride of their own
+    pages = rnd((pages_total + 1, P * (2 * rank + rot) + 8), dtype, seed + 1)[:, : P * (2 * rank + rot)]  # rows with a stride of their own
+    latents = pages[:, : P * rank].unflatten(1, (P, rank))  # the transposed part holds the same latents
+    pages[:, P * rank : 2 * P * rank] = latents.transpose(1, 2).reshape(pages_total + 1, P * rank)
     kv_lens = [p + n for p, n in zip(pasts, lens)]
     positions = [t for n, past in zip(lens, pasts) for t in range(past, past + n)]
     return dict(table=table.cuda(), slots=ints(slot_map), token_seq=ints(token_seq), cu=ints(cu), seq_slots=ints(slots_of),
@@ -134,12 +136,18 @@ def test_latent_kv_write_and_q_rope(dtype, P, rank, rot, rot_dims):
     (4, 40, 12, 3, [33, 2, 1], [5, 0, 17], None),
     (16, 136, 16, 6, [20, 1], [290, 511], 37),
     (32, 520, 64, 2, [3, 1], [250, 100], None),
+    (16, 128, 16, 6, [50, 1, 3], [200, 499, 0], 70),
+    (32, 512, 64, 16, [40, 1, 1], [100, 1900, 333], None),
+    (16, 64, 32, 3, [1, 1, 1, 1], [0, 31, 32, 700], None),
+    (48, 256, 40, 20, [9, 2], [470, 15], 100),
 ])
 def test_latent_attention(dtype, P, rank, rot, H, lens, pasts, window):
     """Mixed steps over scrambled pages against the plain form; the sinks are large enough to count.
-    Queries come in 32-bit and in the cache's type, with the strides that the batched product leaves."""
+    Queries come in 32-bit and in the cache's type, with the strides that the batched product leaves
+    (bfloat16 queries take the matrix-core kernel where it takes the sizes: the last four cases and the
+    first; long pasts are cut into key ranges that are merged)."""
     o = ops()
-    c = latent_case(dtype, P, rank, rot, H, lens, pasts, 21)
+    c = latent_case(dtype, P, rank, rot, H, lens, pasts, 21, pages_total=160)
     N = c["N"]
     sink = rnd((H,), torch.float32, 22, 2.0)
     q_rot = rnd((N, H, rot), torch.float32, 23)
@@ -148,21 +156,27 @@ def test_latent_attention(dtype, P, rank, rot, H, lens, pasts, window):
         args = (q_lat, q_rot, c["pages"], P, rank, rot, c["table"], c["seq_slots"], c["cu"], c["kv_lens"], c["token_seq"],
                 sink, window, 0.11, max(lens), max(c["kv_lens"].tolist()), dtype)
         got = o.latent_attention(*args)
+        on_cores = q_dtype == torch.bfloat16 and rank % 16 == 0 and rank <= 512 and rot % 8 == 0 and P % 16 == 0
+        assert o.last_latent_kernel[0] == ("matrix cores" if on_cores else "generic")
+        if on_cores and max(pasts) > 1000:
+            assert o.last_latent_kernel[1] > 1  # key ranges, merged
         want = REF.latent_attention(*args)
         assert got.shape == (N, H, rank) and (got.double() - want.double()).abs().max() < tol(dtype, 2)
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dtype", DTYPES + ["bfloat16 queries"])
 def test_latent_attention_one_far_key_and_the_sink(dtype):
     """One key far back is made to carry the softmax, then the sink is: the result is that key's
     latent row, then (almost) nothing."""
     o = ops()
     P, rank, rot, H = 16, 64, 8, 2
+    q_dtype = torch.float32 if dtype != "bfloat16 queries" else torch.bfloat16  # (the latter: the matrix-core kernel)
+    dtype = torch.bfloat16 if dtype == "bfloat16 queries" else dtype
     c = latent_case(dtype, P, rank, rot, H, [1], [600], 31)
     far = 3  # position of the key that stands out
     page = int(c["table"][int(c["seq_slots"][0]), far // P])
     row = c["pages"][page, (far % P) * rank : (far % P + 1) * rank].float()
-    q_lat = (row * 40.0 / (row * row).sum()).view(1, 1, rank).repeat(1, H, 1).contiguous()
+    q_lat = (row * 40.0 / (row * row).sum()).view(1, 1, rank).repeat(1, H, 1).contiguous().to(q_dtype)
     q_rot = torch.zeros((1, H, rot), dtype=torch.float32).cuda()
     sink = torch.tensor([-30.0, -30.0]).cuda()
     args = [q_lat, q_rot, c["pages"], P, rank, rot, c["table"], c["seq_slots"], c["cu"], c["kv_lens"], c["token_seq"], sink,

@@ -202,14 +202,24 @@ class TorchOps:
         c = x[:, :rank]
         c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * norm_w.to(self.cd)
         kr = self._rotate_pairs(x[:, rank:], cos_sin, rot_dims)
-        c_pages = pages[:, : page_size * rank].view(-1, page_size, rank)
-        r_pages = pages[:, page_size * rank : page_size * (rank + rot)].view(-1, page_size, rot)
+        c_pages, t_pages, r_pages = self._latent_pages(pages, page_size, rank, rot)
         for n in range(dkv.shape[0]):
             slot = int(slots[n])
             if slot < 0:
                 continue
             c_pages[slot // page_size, slot % page_size] = c[n].to(pages.dtype)
+            t_pages[slot // page_size, :, slot % page_size] = c[n].to(pages.dtype)
             r_pages[slot // page_size, slot % page_size] = kr[n].to(pages.dtype)
+
+    @staticmethod
+    def _latent_pages(pages, P, rank, rot):
+        """Views of a page's three parts: latents [P, rank], the same transposed [rank, P], rotated parts [P, rot]."""
+        n = pages.shape[0]
+        return (pages[:, : P * rank].unflatten(1, (P, rank)), pages[:, P * rank : 2 * P * rank].unflatten(1, (rank, P)),
+                pages[:, 2 * P * rank : P * (2 * rank + rot)].unflatten(1, (P, rot)))
+
+    def latent_query_dtype(self, cache_dtype, page_size, rank, rot):
+        return torch.float32
 
     def latent_q_rope(self, q, cos_sin, rot_dims, heads, dim, rot):
         x = q.view(q.shape[0], heads, dim + rot)[:, :, dim:].to(self.cd)
@@ -224,8 +234,7 @@ class TorchOps:
     def latent_attention(self, q_lat, q_rot, pages, page_size, rank, rot, block_table, seq_slots, cu_tokens, kv_lens,
                          token_seq, sink, window, scale, max_q_len, max_kv_len, out_dtype):
         N, H, _ = q_lat.shape
-        c_pages = pages[:, : page_size * rank].view(-1, page_size, rank)
-        r_pages = pages[:, page_size * rank : page_size * (rank + rot)].view(-1, page_size, rot)
+        c_pages, _, r_pages = self._latent_pages(pages, page_size, rank, rot)
         out = torch.zeros((N, H, rank), dtype=self.cd, device=pages.device)
         for s in range(seq_slots.shape[0]):
             row = int(seq_slots[s])
