@@ -8,6 +8,7 @@
     python bench.py --workload reference-0p6b [--dtype float32]   # the reference's own benchmark shape
     python bench.py --workload mixed-32b [--layers L]             # a prompt chunk beside 63 decoded tokens
     python bench.py --workload serving                            # requests of many lengths arriving over time
+    python bench.py --workload visadra [--sizes small|mid|wide]   # Visadra beside Qwen3 at equal layer sizes, kernel by kernel
 
 A "step" is one decode step of the whole engine (scheduler, model step over the
 paged cache, sampling) with `batch` live requests whose context ends at
@@ -83,6 +84,10 @@ def make_engine(model, batch, context, max_tokens_per_step=8192):
                      max_tokens_per_step=max_tokens_per_step, prefill_chunk=2048, max_pages_per_request=pages_each)
 
 
+def vocab_of(cfg):
+    return cfg.vocab_size if hasattr(cfg, "vocab_size") else cfg.vocab
+
+
 def random_prompts(n, length, vocab, seed):
     import torch
 
@@ -97,7 +102,7 @@ def time_decode(model, cfg, batch, context, steps, warmup):
 
     engine = make_engine(model, batch, context)
     prompt_len = context - (steps + warmup)
-    for p in random_prompts(batch, prompt_len, cfg.vocab_size, 100 + batch):
+    for p in random_prompts(batch, prompt_len, vocab_of(cfg), 100 + batch):
         engine.prefill(engine.add_request(p, steps + warmup + 1))  # each prompt alone, in portions
     for _ in range(warmup):
         engine.step()
@@ -118,7 +123,7 @@ def time_prefill(model, cfg, tokens, repeats=3):
     engine = make_engine(model, 1, tokens + 16, max_tokens_per_step=tokens)
     best = None
     for i in range(repeats + 1):
-        req = engine.add_request(random_prompts(1, tokens, cfg.vocab_size, 7 + i)[0], 1)
+        req = engine.add_request(random_prompts(1, tokens, vocab_of(cfg), 7 + i)[0], 1)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         engine.step()  # the whole prompt in one step, one token drawn
@@ -416,6 +421,168 @@ def more_workloads(steps, warmup):
     return more
 
 
+# ---------------------------------------------------------------------------------------------
+# Visadra (minGRU and latent-attention mixers, dense and routed feed-forwards) beside Qwen3 at
+# equal layer sizes: whole-model prefill and decode, and every kernel of its own beside the like
+# kernel of Qwen3, each against its roofline (bytes it must move at 8 TB/s, or flops at 2.5 PFLOP/s,
+# whichever takes longer).
+# ---------------------------------------------------------------------------------------------
+VISADRA_SIZES = {
+    # width, heads, dim, rot, vdim, rank, minGRU width, dense ff, experts, top, expert ff, shared ff
+    "small": (1024, 8, 64, 32, 64, 256, 1536, 4096, 16, 2, 512, 1024),
+    "mid": (2048, 16, 128, 64, 128, 512, 3072, 8192, 64, 6, 1408, 2816),
+    "wide": (4096, 32, 128, 64, 128, 512, 6144, 12288, 64, 6, 2048, 4096),
+}
+
+
+def visadra_configs(which, groups):
+    """(Visadra config, Qwen3 config of equal width, depth, head count and dense feed-forward)."""
+    from litellmengine_amd.config import Qwen3Config, VisadraConfig
+
+    W, H, dim, rot, vdim, rank, gw, ff, E, top, eff, sff = VISADRA_SIZES[which]
+    att = {"heads": H, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "scale": (dim + rot) ** -0.5,
+           "rot": {"base": 10000.0, "dims": rot}}
+    moe = {"kind": "moe", "router": {"experts": E, "top": top}, "expert": {"ff": eff}, "shared": {"ff": sff}}
+    dense = {"kind": "dense", "ff": ff}
+    four = [{"type": "latent_attention", "mixer": att, "mlp": dense}, {"type": "mingru", "mixer": {"width": gw}, "mlp": moe},
+            {"type": "mingru_2", "mixer": {"width": gw}, "mlp": dense}, {"type": "latent_attention", "mixer": att, "mlp": moe}]
+    v = VisadraConfig.from_dict({"architecture": "Visadra", "vocab": 32768, "width": W, "embedding": {"scale": 1.0},
+                                 "logit_scale": 1.0, "norm": {"eps": 1e-6}, "layers": four * groups})
+    q = Qwen3Config.from_dict(dict(SIZES, num_hidden_layers=4 * groups, hidden_size=W, num_attention_heads=H,
+                                   num_key_value_heads=max(1, H // 4), head_dim=128, intermediate_size=ff, vocab_size=32768))
+    return v, q
+
+
+def timed_launches(launch, repeats=20):
+    import torch
+
+    launch()
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for _ in range(repeats):
+            launch()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / repeats
+        best = dt if best is None else min(best, dt)
+    return best
+
+
+def visadra_kernels(which):
+    """Each kernel of Visadra's own at two shapes (a 2048-token prompt; 8 decoded tokens after 4096) beside
+    the like kernel of Qwen3 at equal sizes: microseconds and the share of its roofline."""
+    import torch
+
+    from litellmengine_amd.csrc.ops import default_ops
+
+    ops = default_ops()
+    W, H, dim, rot, vdim, rank, gw, ff, E, top, eff, sff = VISADRA_SIZES[which]
+    dev, bf = "cuda", torch.bfloat16
+    P = PAGE_SIZE
+    rnd = lambda *shape, dtype=bf, scale=1.0: (torch.randn(shape, device=dev) * scale).to(dtype)
+    ints = lambda values: torch.tensor(values, dtype=torch.int32, device=dev)
+    out = {}
+
+    def entry(name, seconds, flops, nbytes, like=None):
+        floor = max(flops / MFMA_PEAK["bf16"], nbytes / HBM_PEAK)
+        e = {"us": round(seconds * 1e6, 1), "roofline_us": round(floor * 1e6, 2), "frac": round(floor / seconds, 4),
+             "bound": "mfma" if flops / MFMA_PEAK["bf16"] > nbytes / HBM_PEAK else "hbm"}
+        if like is not None:
+            e["like"] = like
+            e["times_farther_from_roofline"] = round(like["frac"] / e["frac"], 2) if e["frac"] > 0 else None
+        out[name] = e
+        return e
+
+    for shape, S, q_len, past in (("prefill_2048", 1, 2048, 0), ("decode_b8_ctx4096", 8, 1, 4095)):
+        N, kv = S * q_len, past + q_len
+        pages_each = -(-kv // P)
+        table = torch.arange(S * pages_each, dtype=torch.int32, device=dev).view(S, pages_each).contiguous()
+        seq_slots, cu = ints(list(range(S))), ints([i * q_len for i in range(S + 1)])
+        kv_lens = ints([kv] * S)
+        token_seq = ints([i // q_len for i in range(N)])
+        visible = S * (q_len * past + q_len * (q_len + 1) / 2)  # (query, key) pairs
+        # latent attention beside grouped-query attention
+        lat_pages = rnd(S * pages_each + 1, P * (2 * rank + rot))
+        q_lat, q_rot = rnd(H, N, rank, scale=0.1).transpose(0, 1), rnd(N, H, rot, dtype=torch.float32, scale=0.1)
+        sink = torch.zeros(H, device=dev)
+        t = timed_launches(lambda: ops.latent_attention(q_lat, q_rot, lat_pages, P, rank, rot, table, seq_slots, cu, kv_lens,
+                                                        token_seq, sink, None, 0.1, q_len, kv, bf))
+        nkv, d = max(1, H // 4), 128
+        kv_layer = rnd(S * pages_each + 1, 2, nkv, P, d)
+        q = rnd(N, H, d, scale=0.1)
+        tq = timed_launches(lambda: ops.paged_attention(q, kv_layer, table, seq_slots, cu, kv_lens, token_seq, None, 0.1,
+                                                        q_len, q_len, kv))
+        like = entry(f"{shape}/paged_attention (Qwen3)", tq, 4.0 * H * d * visible, 2.0 * (S * kv * 2 * nkv * d + 2 * N * H * d))
+        entry(f"{shape}/latent_attention", t, 2.0 * H * (2 * rank + rot) * visible,
+              2.0 * (S * kv * (2 * rank + rot) + 2 * N * H * rank), dict(like, name="paged_attention"))
+        # the latents' and keys' way into the pages
+        dkv, nw = rnd(N, rank + rot), torch.ones(rank, device=dev, dtype=bf)
+        cos_sin = ops.rope_table(ints([past + i % q_len for i in range(N)]), torch.ones(rot // 2, device=dev))
+        slots = ints([int(table[i // q_len, (past + i % q_len) // P]) * P + (past + i % q_len) % P for i in range(N)]) if N <= 64 else \
+            (table.long()[:, : pages_each].repeat_interleave(P, 1)[:, past:kv] * P + torch.arange(past, kv, device=dev) % P).reshape(-1).int()
+        t = timed_launches(lambda: ops.latent_kv_write(dkv, nw, 1e-6, cos_sin, rot, slots, lat_pages, P, rank, rot))
+        qkv = rnd(N, (H + 2 * nkv) * d)
+        cs2 = ops.rope_table(ints([past + i % q_len for i in range(N)]), torch.ones(d // 2, device=dev))
+        one = torch.ones(d, device=dev, dtype=bf)
+        tq = timed_launches(lambda: ops.qk_norm_rope_write(qkv, slots, one, one, cs2, d, 1e-6, kv_layer, H, nkv, d))
+        like = entry(f"{shape}/qk_norm_rope_write (Qwen3)", tq, 0, 2.0 * N * (2 * H + 4 * nkv) * d)
+        entry(f"{shape}/latent_kv_write", t, 0, 2.0 * N * (3 * rank + 2 * rot), dict(like, name="qk_norm_rope_write"))
+        # the recurrence: nothing like it in Qwen3; beside the residual add + norm, which moves rows as it does
+        zxg, bias = rnd(N, 3 * gw, dtype=torch.float32), torch.zeros(gw, device=dev)
+        state = torch.zeros(S + 1, gw, device=dev)
+        t = timed_launches(lambda: ops.mingru_scan(zxg, bias, bias, state, seq_slots, cu, bf, q_len))
+        hidden, delta, w = rnd(N, W, dtype=torch.float32), rnd(N, W), torch.ones(W, device=dev, dtype=bf)
+        tq = timed_launches(lambda: ops.add_rmsnorm(hidden, delta, w, 1e-6, bf))
+        like = entry(f"{shape}/add_rmsnorm (Qwen3)", tq, 0, N * W * (4 + 4 + 2 + 2.0))
+        entry(f"{shape}/mingru_scan", t, 0, N * gw * (12 + 2.0), dict(like, name="add_rmsnorm"))
+        t = timed_launches(lambda: ops.rmsnorm_add(hidden, delta, w, 1e-6, bf))
+        entry(f"{shape}/rmsnorm_add", t, 0, N * W * (4 + 4 + 2 + 2.0), dict(like, name="add_rmsnorm"))
+        # the routed experts beside the dense gated feed-forward (its two products and the activation)
+        x = rnd(N, W, scale=0.1)
+        gate_up, down = rnd(E, 2 * eff, W, scale=0.02), rnd(E, W, eff, scale=0.02)
+        ids, gains = ops.moe_route(rnd(N, E, dtype=torch.float32), torch.zeros(E, device=dev), top)
+        t = timed_launches(lambda: ops.moe_experts(x, ids, gains, gate_up, down), repeats=5)
+        used = min(E, N * top)
+        wgu, wd = rnd(2 * ff, W, scale=0.02), rnd(W, ff, scale=0.02)
+        tq = timed_launches(lambda: ops.linear(ops.gate_up_silu(x, wgu), wd), repeats=5)
+        like = entry(f"{shape}/gated feed-forward (Qwen3)", tq, 6.0 * N * W * ff, 2.0 * (3 * W * ff + 2 * N * W))
+        entry(f"{shape}/moe_experts", t, 6.0 * N * top * W * eff, 2.0 * (3 * used * W * eff + 2 * N * W),
+              dict(like, name="gated feed-forward"))
+        del lat_pages, kv_layer
+    return out
+
+
+def visadra_workload(args):
+    import torch
+
+    from litellmengine_amd.models import random_model
+
+    which = args.sizes if args.sizes in VISADRA_SIZES else "mid"
+    groups = max(1, args.layers // 4) if args.layers != SIZES["num_hidden_layers"] else 2
+    vcfg, qcfg = visadra_configs(which, groups)
+    line = {"metric": f"Visadra beside Qwen3 at equal layer sizes ({which}): prefill tok/s @ 2048 and decode tok/s @ batch "
+                      f"{args.batch}, context {args.context}", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+            "data": "synthetic: seeded random weights, uniform random token ids", "higher_is_better": True,
+            "config": {"sizes": dict(zip(("width", "heads", "dim", "rot_dim", "vdim", "kv_rank", "mingru_width", "dense_ff",
+                                          "experts", "top", "expert_ff", "shared_ff"), VISADRA_SIZES[which])),
+                       "layers": 4 * groups, "pattern": "latent+dense, mingru+moe, mingru+dense, latent+moe"}}
+    steps, warmup = min(args.steps, 16), min(args.warmup, 4)
+    for name, cfg in (("visadra", vcfg), ("qwen3", qcfg)):
+        model = random_model(cfg, seed=0, dtype="bfloat16")
+        dt = time_decode(model, cfg, args.batch, args.context, steps, warmup)
+        pt = time_prefill(model, cfg, PREFILL_TOKENS)
+        line[name] = {"decode_tok_s": round(args.batch / dt, 1), "decode_ms_per_step": round(dt * 1e3, 3),
+                      "prefill_tok_s": round(PREFILL_TOKENS / pt, 1), "prefill_ms": round(pt * 1e3, 3)}
+        del model
+        torch.cuda.empty_cache()
+    line["value"] = line["visadra"]["decode_tok_s"]
+    line["steps"], line["warmup"] = steps, warmup
+    line["kernels"] = visadra_kernels(which)
+    print(json.dumps(line))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -427,11 +594,13 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--no-more", action="store_true", help="skip the other workloads that the default line carries")
-    ap.add_argument("--sizes", default="8b", choices=["8b", "0p6b", "32b"],
-                    help="layer sizes of the decode workload: Qwen3-8B (default, the headline), Qwen3-0.6B or Qwen3-32B")
-    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving"],
+    ap.add_argument("--sizes", default="8b", choices=["8b", "0p6b", "32b", "small", "mid", "wide"],
+                    help="layer sizes of the decode workload: Qwen3-8B (default, the headline), Qwen3-0.6B or Qwen3-32B; "
+                         "small, mid or wide: the layer sizes of --workload visadra")
+    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving", "visadra"],
                     help="decode (default: the headline line), the reference's own benchmark shape at Qwen3-0.6B "
-                         "sizes, or a mixed prompt-portion + decode step at Qwen3-32B sizes")
+                         "sizes, a mixed prompt-portion + decode step at Qwen3-32B sizes, requests arriving over time, "
+                         "or Visadra beside Qwen3 at equal layer sizes with every kernel against its roofline")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported")
@@ -445,6 +614,8 @@ def main():
             return reference_workload(args)
         if args.workload == "serving":
             return serving_workload(args)
+        if args.workload == "visadra":
+            return visadra_workload(args)
         args.steps, args.warmup = min(args.steps, 3), min(args.warmup, 1)
         return mixed_workload(args)
 

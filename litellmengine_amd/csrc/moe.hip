@@ -5,11 +5,12 @@
 //   act[p]   = silu(Wg[e_p] x_n) * (Wu[e_p] x_n)      p = (token n, k-th choice)      moe_gate_up
 //   out[n]   = sum_k gains[n, k] * Wd[e_(n,k)] act[(n, k)]        32-bit              moe_down
 //
-// Few tokens (decoding): every (token, choice) pair streams the rows of its expert's weights, a
-// wavefront per output element.  Many tokens (prompt portions): the pairs are first put in the order of
-// their experts (a counting sort on the device), then tiles of 16 pairs of one expert go through the
-// matrix cores against that expert's weights (moe_*_tile kernels, bfloat16), so that an expert's
-// weights are read once per tile and not once per token.
+// Few tokens (decoding), or float32: every (token, choice) pair streams the rows of its expert's
+// weights, a wavefront per output element.  Many bfloat16 tokens (prompt portions, large batches): the
+// pairs are first put in the order of their experts (a counting sort on the device), then tiles of 64
+// pairs of one expert go through the matrix cores against that expert's weights (moe_*_tile kernels),
+// so that an expert's weights are read once per tile and not once per token; the per-pair results
+// are added up per token, in the order of its choices, by a last kernel.
 #include "common.h"
 
 LLE_DEFINE_ERROR_STRING()
@@ -122,5 +123,239 @@ extern "C" int lle_moe_experts(const void* x, const void* ids, const void* gains
         moe_down_kernel<bf16_t><<<g2, 256, 0, stream>>>((const bf16_t*)act, (const int32_t*)ids, (const float*)gains,
                                                          (const bf16_t*)down, (float*)out, top, F, H);
     }
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Many pairs: sorted by expert, then tiles on the matrix cores (bfloat16).
+//   counts[e]            pairs of expert e                                   moe_count_kernel
+//   first[e], tile0[e]   first sorted row / first 64-row tile of expert e    moe_plan_kernel (one workgroup)
+//   order[row] = pair, place[pair] = row                                     moe_place_kernel
+// The order of an expert's pairs among themselves is whatever the atomics give; no value depends on it.
+// A tile workgroup finds its expert by walking tile0[] (at most 256 experts), and leaves if the step
+// has fewer tiles than the grid (the grid is sized for the worst case, pairs / 64 + experts).
+// Products as C^T = W X^T with v_mfma_f32_16x16x32_bf16: lane (c = lane / 16, r = lane % 16) loads 16
+// bytes of row r of a 16-row tile of W (A) and of X (B) and holds outputs n = 4c .. 4c + 3 of row r.
+// A wavefront keeps 64 rows x 64 outputs (gate_up: 64 rows x 32 gate + 32 up); four wavefronts of a
+// workgroup sit side by side along the outputs and share the X rows through the cache.
+// ---------------------------------------------------------------------------------------------
+#define MOE_TM 64
+typedef bf16_t mbf16x8 __attribute__((ext_vector_type(8)));
+typedef bf16_t mbf16x4 __attribute__((ext_vector_type(4)));
+typedef float mf32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void moe_zero_kernel(int32_t* __restrict__ p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void moe_count_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ counts,
+                                                         int pairs) {
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p < pairs) atomicAdd(&counts[ids[p]], 1);
+}
+
+// plan = [counts E | cursor E | first E | tile0 E + 1]
+__global__ __launch_bounds__(64) void moe_plan_kernel(int32_t* __restrict__ plan, int E) {
+    if (threadIdx.x != 0) return;
+    int32_t* counts = plan;
+    int32_t* first = plan + 2 * E;
+    int32_t* tile0 = plan + 3 * E;
+    int row = 0, tile = 0;
+    for (int e = 0; e < E; ++e) {
+        first[e] = row;
+        tile0[e] = tile;
+        row += counts[e];
+        tile += (counts[e] + MOE_TM - 1) / MOE_TM;
+    }
+    tile0[E] = tile;
+}
+
+__global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ plan,
+                                                         int32_t* __restrict__ order, int32_t* __restrict__ place,
+                                                         int pairs, int E) {
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= pairs) return;
+    const int e = ids[p];
+    const int row = plan[2 * E + e] + atomicAdd(&plan[E + e], 1);
+    order[row] = p;
+    place[p] = row;
+}
+
+struct MoeTile {
+    int expert, row0, rows;  // rows [row0, row0 + rows) of the sorted order, all of `expert`
+};
+
+__device__ __forceinline__ bool moe_find_tile(const int32_t* __restrict__ plan, int E, int tile, MoeTile& t) {
+    const int32_t* counts = plan;
+    const int32_t* first = plan + 2 * E;
+    const int32_t* tile0 = plan + 3 * E;
+    if (tile >= tile0[E]) return false;
+    int e = 0;
+    while (tile0[e + 1] <= tile) ++e;
+    t.expert = e;
+    const int within = (tile - tile0[e]) * MOE_TM;
+    t.row0 = first[e] + within;
+    t.rows = min(MOE_TM, counts[e] - within);
+    return true;
+}
+
+// act[row, f] = silu(x Wg^T) * (x Wu^T) for the sorted rows; grid (tiles, ceil(F / 128)), 4 wavefronts of 32 f each
+__global__ __launch_bounds__(256) void moe_gate_up_tile_kernel(const bf16_t* __restrict__ x,
+                                                                const int32_t* __restrict__ plan,
+                                                                const int32_t* __restrict__ order,
+                                                                const bf16_t* __restrict__ gate_up,
+                                                                bf16_t* __restrict__ act, int E, int top, int F, int K) {
+    MoeTile t;
+    if (!moe_find_tile(plan, E, blockIdx.x, t)) return;
+    const int lane = threadIdx.x % LLE_WAVE, c = lane / 16, r = lane % 16;
+    const int f0 = (blockIdx.y * 4 + threadIdx.x / LLE_WAVE) * 32;
+    if (f0 >= F) return;
+    const bf16_t* xr[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int row = mt * 16 + r;
+        xr[mt] = row < t.rows ? x + (int64_t)(order[t.row0 + row] / top) * K : nullptr;
+    }
+    const bf16_t* w = gate_up + (int64_t)t.expert * 2 * F * K;
+    const bf16_t* wr[4];  // gate rows f0 + r, f0 + 16 + r, then the up rows of the same f
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+        const int f = f0 + (nt % 2) * 16 + r;
+        wr[nt] = f < F ? w + (int64_t)((nt / 2) * F + f) * K : nullptr;
+    }
+    mf32x4 acc[4][4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mf32x4{0.f, 0.f, 0.f, 0.f};
+    mbf16x8 zero;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) zero[i] = (bf16_t)0.0f;
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const int k = k0 + 8 * c;
+        mbf16x8 a[4], b[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) a[nt] = (wr[nt] && k < K) ? *(const mbf16x8*)(wr[nt] + k) : zero;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) b[mt] = (xr[mt] && k < K) ? *(const mbf16x8*)(xr[mt] + k) : zero;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[nt][mt], 0, 0, 0);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int row = mt * 16 + r;
+        if (row >= t.rows) continue;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int f = f0 + half * 16 + 4 * c;
+            if (f >= F) continue;  // (F is a multiple of 4: whole groups)
+            mbf16x4 v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float g = acc[half][mt][i], u = acc[2 + half][mt][i];
+                v[i] = (bf16_t)(g / (1.0f + expf(-g)) * u);
+            }
+            *(mbf16x4*)(act + (int64_t)(t.row0 + row) * F + f) = v;
+        }
+    }
+}
+
+// y[row, o] = act[row] Wd[e]^T for the sorted rows, float32; grid (tiles, ceil(H / 256)), 4 wavefronts of 64 o each
+__global__ __launch_bounds__(256) void moe_down_tile_kernel(const bf16_t* __restrict__ act,
+                                                             const int32_t* __restrict__ plan,
+                                                             const bf16_t* __restrict__ down, float* __restrict__ y,
+                                                             int E, int F, int H) {
+    MoeTile t;
+    if (!moe_find_tile(plan, E, blockIdx.x, t)) return;
+    const int lane = threadIdx.x % LLE_WAVE, c = lane / 16, r = lane % 16;
+    const int o0 = (blockIdx.y * 4 + threadIdx.x / LLE_WAVE) * 64;
+    if (o0 >= H) return;
+    const bf16_t* xr[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int row = mt * 16 + r;
+        xr[mt] = row < t.rows ? act + (int64_t)(t.row0 + row) * F : nullptr;
+    }
+    const bf16_t* wr[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+        const int o = o0 + nt * 16 + r;
+        wr[nt] = o < H ? down + ((int64_t)t.expert * H + o) * F : nullptr;
+    }
+    mf32x4 acc[4][4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mf32x4{0.f, 0.f, 0.f, 0.f};
+    mbf16x8 zero;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) zero[i] = (bf16_t)0.0f;
+    for (int k0 = 0; k0 < F; k0 += 32) {
+        const int k = k0 + 8 * c;
+        mbf16x8 a[4], b[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) a[nt] = (wr[nt] && k < F) ? *(const mbf16x8*)(wr[nt] + k) : zero;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) b[mt] = (xr[mt] && k < F) ? *(const mbf16x8*)(xr[mt] + k) : zero;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[nt][mt], 0, 0, 0);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int row = mt * 16 + r;
+        if (row >= t.rows) continue;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            const int o = o0 + nt * 16 + 4 * c;
+            if (o < H) *(mf32x4*)(y + (int64_t)(t.row0 + row) * H + o) = acc[nt][mt];  // (H is a multiple of 4)
+        }
+    }
+}
+
+// out[n, :] = sum_k gains[n, k] * y[place[n top + k], :], in the order of k
+__global__ __launch_bounds__(256) void moe_gather_kernel(const float* __restrict__ y, const int32_t* __restrict__ place,
+                                                          const float* __restrict__ gains, float* __restrict__ out,
+                                                          int top, int H) {
+    const int n = blockIdx.x;
+    for (int o = threadIdx.x * 4; o < H; o += blockDim.x * 4) {
+        mf32x4 total = mf32x4{0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < top; ++k) {
+            const int p = n * top + k;
+            total += gains[p] * *(const mf32x4*)(y + (int64_t)place[p] * H + o);
+        }
+        *(mf32x4*)(out + (int64_t)n * H + o) = total;
+    }
+}
+
+extern "C" int lle_moe_tile_rows(void) { return MOE_TM; }
+
+// bfloat16, K and F multiples of 8, H a multiple of 4, E <= 256.  Scratch: plan int32 [4 E + 1], order and
+// place int32 [N top], act bfloat16 [N top, F], y float32 [N top, H].
+extern "C" int lle_moe_experts_tiled(const void* x, const void* ids, const void* gains, const void* gate_up,
+                                     const void* down, void* plan, void* order, void* place, void* act, void* y,
+                                     void* out, int N, int top, int E, int F, int K, int H, hipStream_t stream) {
+    if (N <= 0) return 0;
+    const int64_t pairs64 = (int64_t)N * top;
+    if (top <= 0 || E <= 0 || E > 256 || K % 8 || F % 8 || H % 4 || pairs64 > 0x3fffffff) return (int)hipErrorInvalidValue;
+    const int pairs = (int)pairs64;
+    const int tiles = pairs / MOE_TM + E;  // at most: every expert leaves one tile partly empty
+    moe_zero_kernel<<<(2 * E + 255) / 256, 256, 0, stream>>>((int32_t*)plan, 2 * E);
+    moe_count_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>((const int32_t*)ids, (int32_t*)plan, pairs);
+    moe_plan_kernel<<<1, 64, 0, stream>>>((int32_t*)plan, E);
+    moe_place_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>((const int32_t*)ids, (int32_t*)plan, (int32_t*)order,
+                                                               (int32_t*)place, pairs, E);
+    moe_gate_up_tile_kernel<<<dim3(tiles, (F + 127) / 128), 256, 0, stream>>>(
+        (const bf16_t*)x, (const int32_t*)plan, (const int32_t*)order, (const bf16_t*)gate_up, (bf16_t*)act, E, top, F, K);
+    moe_down_tile_kernel<<<dim3(tiles, (H + 255) / 256), 256, 0, stream>>>((const bf16_t*)act, (const int32_t*)plan,
+                                                                            (const bf16_t*)down, (float*)y, E, F, H);
+    moe_gather_kernel<<<N, 256, 0, stream>>>((const float*)y, (const int32_t*)place, (const float*)gains, (float*)out,
+                                                top, H);
     LLE_RETURN_LAUNCH_STATUS();
 }

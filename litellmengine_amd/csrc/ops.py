@@ -716,7 +716,7 @@ class HipOps:
         return hidden if out is None else out
 
     # -- gated recurrence -------------------------------------------------------------
-    MINGRU_PIECE = 64  # tokens of one request that one thread walks before the walk is cut into pieces
+    MINGRU_PIECE = 16  # tokens of one request that one thread walks before the walk is cut into pieces
 
     def mingru_scan(self, zxg, z_bias, x_bias, state, seq_slots, cu_tokens, out_dtype, max_q_len: int = 0):
         """zxg [N, 3 W] (update-gate, candidate and output-gate inputs side by side; float32 or bfloat16),
@@ -891,9 +891,13 @@ class HipOps:
                   _ptr(gains), N, E, top)
         return ids, gains
 
+    MOE_TILED_MIN_PAIRS = 129  # (token, choice) pairs from which the sorted, tiled kernels take a bfloat16 step
+
     def moe_experts(self, x, ids, gains, gate_up, down) -> torch.Tensor:
         """x [N, K]; ids, gains [N, top]; gate_up [E, 2 F, K] (gate rows, then up rows); down [E, H, F] ->
-        float32 [N, H]: sum_k gains[n, k] * down[e] (silu(gate[e] x) * (up[e] x)), e = ids[n, k]."""
+        float32 [N, H]: sum_k gains[n, k] * down[e] (silu(gate[e] x) * (up[e] x)), e = ids[n, k].
+        Few pairs, or float32: every pair streams its expert's rows.  Many bfloat16 pairs: sorted by expert
+        on the device, then tiles of 64 pairs of one expert on the matrix cores."""
         _dev(x, "x")
         _dev(ids, "ids", torch.int32)
         _dev(gains, "gains", torch.float32)
@@ -907,6 +911,16 @@ class HipOps:
         _need(gate_up.shape == (E, F2, K) and F2 % 2 == 0 and down.shape == (E, H, F2 // 2), "expert weights do not fit")
         act = torch.empty((N * top, F2 // 2), dtype=x.dtype, device=x.device)
         out = torch.empty((N, H), dtype=torch.float32, device=x.device)
+        F = F2 // 2
+        if (x.dtype == torch.bfloat16 and N * top >= self.MOE_TILED_MIN_PAIRS and E <= 256 and K % 8 == 0 and F % 8 == 0
+                and H % 4 == 0):
+            plan = torch.empty((4 * E + 1,), dtype=torch.int32, device=x.device)
+            order = torch.empty((2, N * top), dtype=torch.int32, device=x.device)
+            y = torch.empty((N * top, H), dtype=torch.float32, device=x.device)
+            self._run("moe", "lle_moe_experts_tiled", [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+                      _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(plan), order[0].data_ptr(),
+                      order[1].data_ptr(), _ptr(act), _ptr(y), _ptr(out), N, top, E, F, K, H)
+            return out
         self._run("moe", "lle_moe_experts", [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
                   _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(act), _ptr(out), N, top, F2 // 2,
                   K, H, dtype_code(x.dtype))

@@ -222,8 +222,11 @@ def test_moe_route_picks_the_largest_and_the_lower_index_among_equals():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("N,K,F,H,E,top", [(1, 72, 40, 72, 5, 2), (37, 200, 24, 200, 9, 3), (4, 64, 130, 64, 3, 3),
-                                           (300, 128, 64, 128, 8, 2)])
+                                           (300, 128, 64, 128, 8, 2), (70, 200, 24, 204, 9, 3), (513, 96, 136, 100, 40, 6),
+                                           (200, 64, 8, 64, 2, 1)])
 def test_moe_experts(dtype, N, K, F, H, E, top):
+    """Few pairs stream their experts' rows; from 129 bfloat16 pairs on they are sorted by expert and go through
+    the matrix cores in tiles (the last four cases; experts with no pair, with one, with more than a tile)."""
     o = ops()
     x = rnd((N, K), dtype, 61)
     gate_up = rnd((E, 2 * F, K), dtype, 62, 0.2)
