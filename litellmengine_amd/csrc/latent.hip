@@ -224,24 +224,32 @@ extern "C" int lle_latent_attention_generic(const void* q_lat, int q_lat_dtype, 
 
 // ---------------------------------------------------------------------------------------------
 // bfloat16 on the matrix cores.  The rows of a request are its (token, head) pairs, token after
-// token; a wavefront takes one tile of 16 rows over a range of 32-key steps:
-//   S^T = K Q^T      A = [16 keys x 32 elements] of [c | k_rot], B = the queries (in registers)
-//   O^T += C^T P^T   A = [16 latent elements x 32 keys] of the transposed latents, B = P^T
+// token; a workgroup of four wavefronts takes one tile of 16 rows over a range of 64-key steps:
+//   S^T = K Q^T      A = [16 keys x 32 elements] of [c | k_rot], B = the queries (in LDS):
+//                    wavefront w takes the keys 16 w .. 16 w + 15 of the step
+//   O^T += C^T P^T   A = [16 latent elements x 32 keys] of the transposed latents, B = P^T:
+//                    wavefront w takes a quarter of the latent's elements over all 64 keys
 // With v_mfma_f32_16x16x32_bf16 lane (c = lane / 16, r = lane % 16) holds of a result tile column r,
-// rows 4c .. 4c + 3.  Row q of K tile x stands for key 8 (q / 4) + 4 x + q % 4 of the step, so the
-// lane's eight scores are the consecutive keys 8c .. 8c + 7 of query row r: the B operand of the
-// second product as it stands, and its A operand is one 16-byte piece of the transposed page.
-// The softmax state of row r lives in the four lanes r + 16c.  Every operand comes straight from
-// the pages (no LDS: wavefronts are independent, one per workgroup).  With `nsplit` > 1 a tile's
-// keys are cut into ranges whose unnormalised results (and m, l) go to a workspace and are merged
-// by latent_combine_kernel; the sink (m = sink, l = 1) belongs to the first range.
+// rows 4c .. 4c + 3: four keys of query row r after the first product.  The rows' maxima and the
+// weights P (bfloat16, [row][key]) cross between the wavefronts through LDS, two barriers a step;
+// the buffers take turns, so a step's writes never meet the reads of the step before.  All of a
+// step's operands (one K tile and the wavefront's share of the transposed latents) are asked for
+// at the top of the step, straight from the pages, and travel together.  The quarter of the
+// accumulators per wavefront is what leaves registers for that.  With `nsplit` > 1 a tile's keys
+// are cut into ranges whose unnormalised results (and m, l) go to a workspace and are merged by
+// latent_combine_kernel; the sink (m = sink, l = 1) belongs to the first range.
 // RK = 32-element steps over the latent (rank <= 32 RK, padded with zeros), RR the same for k_rot.
+// PAD: rank < 32 RK or rot < 32 RR, and the operands' tails are filled with zeros under a condition.
+// Without it every load is unconditional (a key outside the tile's range is read from the nearest one
+// inside it and masked afterwards; the pages hold finite numbers everywhere).
 // ---------------------------------------------------------------------------------------------
 typedef bf16_t lbf16x8 __attribute__((ext_vector_type(8)));
 typedef bf16_t lbf16x4 __attribute__((ext_vector_type(4)));
 typedef float lf32x4 __attribute__((ext_vector_type(4)));
 #define LAT_NEG_BIG (-1.0e30f)
 #define LAT_LOG2E 1.4426950408889634f
+#define LAT_STEP 64
+#define LAT_P_STRIDE 72  // bfloat16 elements between the rows of P in LDS: 64 keys and 16 bytes to spread the banks
 
 __device__ __forceinline__ lbf16x8 lat_zero8() {
     lbf16x8 z;
@@ -250,22 +258,28 @@ __device__ __forceinline__ lbf16x8 lat_zero8() {
     return z;
 }
 
-template <int RK, int RR>
-__global__ __launch_bounds__(64) void latent_attention_mfma_kernel(
+template <int RK, int RR, bool PAD>
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ q_lat, int64_t ql_stride_n, int64_t ql_stride_h, const float* __restrict__ q_rot,
     const bf16_t* __restrict__ pages, int64_t page_stride, int P, int rank, int rot,
     const int32_t* __restrict__ block_table, int max_pages, const int32_t* __restrict__ seq_slots,
     const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ kv_lens, const float* __restrict__ sink,
     int window, float scale, bf16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml, int H,
     int tiles_max, int nsplit) {
-    const int lane = threadIdx.x, c = lane / 16, r = lane % 16;
+    constexpr int NT = RK / 2;  // value tiles (16 latent elements each) of one wavefront, of 2 RK
+    __shared__ float s_max[2][4][16];
+    __shared__ __attribute__((aligned(16))) bf16_t s_p[2][16][LAT_P_STRIDE];
+    __shared__ float s_l[4][16];
+    __shared__ __attribute__((aligned(16))) bf16_t s_q[16][32 * (RK + RR) + 8];  // (8 more: rows 16 bytes off the banks)
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE, c = lane / 16, r = lane % 16;
     int item = blockIdx.x;
     const int split = item % nsplit;
     item /= nsplit;
-    const int tile = item % tiles_max, s = item / tiles_max;
+    // the last tiles of a request see the most keys: they start first, so that no long tile is left for the end
+    const int tile = tiles_max - 1 - item % tiles_max, s = item / tiles_max;
     const int q0 = cu_tokens[s], q_len = cu_tokens[s + 1] - q0;
     const int rows = q_len * H;
-    if (tile * 16 >= rows) return;  // (the whole wavefront)
+    if (tile * 16 >= rows) return;  // (the whole workgroup)
     const int past = kv_lens[s] - q_len;
     const int rho = tile * 16 + r;
     const bool valid = rho < rows;
@@ -277,140 +291,166 @@ __global__ __launch_bounds__(64) void latent_attention_mfma_kernel(
     const int lo_min = window > 0 ? max(0, past + t_first - window + 1) : 0;
     const int32_t* table = block_table + (int64_t)seq_slots[s] * max_pages;
 
-    lbf16x8 qv[RK + RR];
+    // the tile's queries wait in LDS as the B operands of the first product: row r, elements 32 i + 8 c .. + 7
+    // for lane (c, r) and step i; every wavefront writes a quarter of the steps and reads them all
     {
         const bf16_t* ql = q_lat + (int64_t)(q0 + t) * ql_stride_n + (int64_t)h * ql_stride_h;
-#pragma unroll
-        for (int ks = 0; ks < RK; ++ks) {
-            const int e0 = 32 * ks + 8 * c;
-            qv[ks] = (valid && e0 < rank) ? *(const lbf16x8*)(ql + e0) : lat_zero8();
-        }
         const float* qr = q_rot + ((int64_t)(q0 + t) * H + h) * rot;
-#pragma unroll
-        for (int kr = 0; kr < RR; ++kr) {
-            const int e0 = 32 * kr + 8 * c;
+        for (int i = wave; i < RK + RR; i += 4) {
             lbf16x8 v = lat_zero8();
-            if (valid && e0 < rot) {
+            if (i < RK) {
+                const int e0 = 32 * i + 8 * c;
+                if (valid && e0 < rank) v = *(const lbf16x8*)(ql + e0);
+            } else {
+                const int e0 = 32 * (i - RK) + 8 * c;
+                if (valid && e0 < rot) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[i] = (bf16_t)qr[e0 + i];
+                    for (int e = 0; e < 8; ++e) v[e] = (bf16_t)qr[e0 + e];
+                }
             }
-            qv[RK + kr] = v;
+            *(lbf16x8*)&s_q[r][32 * i + 8 * c] = v;
         }
     }
-    lf32x4 o[2 * RK];
+    __syncthreads();
+    lf32x4 o[NT];
 #pragma unroll
-    for (int n = 0; n < 2 * RK; ++n) o[n] = lf32x4{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < NT; ++i) o[i] = lf32x4{0.f, 0.f, 0.f, 0.f};
     const bool first = split == 0 && valid;
-    float m = first ? sink[h] * LAT_LOG2E : LAT_NEG_BIG;  // base 2
-    float l = (first && c == 0) ? 1.0f : 0.0f;            // this lane's share of the row's sum
+    float m = first ? sink[h] * LAT_LOG2E : LAT_NEG_BIG;     // base 2; the same in the row's lanes of every wavefront
+    float l = (first && c == 0 && wave == 0) ? 1.0f : 0.0f;  // this lane's share of the row's sum
     const float sc2 = scale * LAT_LOG2E;
 
-    const int s_begin = lo_min / 32, s_end = kmax / 32 + 1;
+    const int s_begin = lo_min / LAT_STEP, s_end = kmax / LAT_STEP + 1;
     const int per = (s_end - s_begin + nsplit - 1) / nsplit;
     const int st_lo = s_begin + split * per, st_hi = min(s_end, st_lo + per);
-    for (int st = st_lo; st < st_hi; ++st) {
-        const int j0 = st * 32;
-        lf32x4 sacc[2];
+    int buf = 0;
+    for (int st = st_lo; st < st_hi; ++st, buf ^= 1) {
+        const int j0 = st * LAT_STEP;
+        // every operand of the step is asked for here
+        lbf16x8 ka[RK + RR];
+        {
+            const int key = min(max(j0 + 16 * wave + r, lo_min), kmax);  // (outside: masked below)
+            const bf16_t* pg = pages + (int64_t)table[key / P] * page_stride;
+            const bf16_t* kp = pg + (int64_t)(key % P) * rank + 8 * c;
+            const bf16_t* krp = pg + (int64_t)2 * P * rank + (int64_t)(key % P) * rot + 8 * c;
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            sacc[x] = lf32x4{0.f, 0.f, 0.f, 0.f};
-            const int key = j0 + 8 * (r / 4) + 4 * x + r % 4;
-            const bool ok = key >= lo_min && key <= kmax;
-            const bf16_t* pg = pages + (int64_t)(ok ? table[key / P] : 0) * page_stride;
-            const bf16_t* kp = pg + (int64_t)(key % P) * rank;
-            const bf16_t* krp = pg + (int64_t)2 * P * rank + (int64_t)(key % P) * rot;
+            for (int ks = 0; ks < RK; ++ks)
+                ka[ks] = (!PAD || 32 * ks + 8 * c < rank) ? *(const lbf16x8*)(kp + 32 * ks) : lat_zero8();
 #pragma unroll
-            for (int ks = 0; ks < RK; ++ks) {
-                const int e0 = 32 * ks + 8 * c;
-                const lbf16x8 a = (ok && e0 < rank) ? *(const lbf16x8*)(kp + e0) : lat_zero8();
-                sacc[x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qv[ks], sacc[x], 0, 0, 0);
-            }
+            for (int kr = 0; kr < RR; ++kr)
+                ka[RK + kr] = (!PAD || 32 * kr + 8 * c < rot) ? *(const lbf16x8*)(krp + 32 * kr) : lat_zero8();
+        }
+        lbf16x8 va[2][NT];
 #pragma unroll
-            for (int kr = 0; kr < RR; ++kr) {
-                const int e0 = 32 * kr + 8 * c;
-                const lbf16x8 a = (ok && e0 < rot) ? *(const lbf16x8*)(krp + e0) : lat_zero8();
-                sacc[x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qv[RK + kr], sacc[x], 0, 0, 0);
+        for (int kk = 0; kk < 2; ++kk) {
+            // this lane's eight keys, inside one page; a group outside the tile's range has no weight and is
+            // read from the nearest group inside it
+            const int gkey = min(max(j0 + 32 * kk + 8 * c, lo_min & ~7), kmax & ~7);
+            const bf16_t* vt = pages + (int64_t)table[gkey / P] * page_stride + (int64_t)P * rank + gkey % P;
+#pragma unroll
+            for (int i = 0; i < NT; ++i) {
+                const int n = wave * NT + i;
+                va[kk][i] = (!PAD || 16 * n < rank) ? *(const lbf16x8*)(vt + (int64_t)(16 * n + r) * P) : lat_zero8();
             }
         }
-        float sv[8];
+        lf32x4 sacc = lf32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < RK + RR; ++i)
+            sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[i], *(const lbf16x8*)&s_q[r][32 * i + 8 * c], sacc, 0, 0, 0);
+        float sv[4];
         float mx = LAT_NEG_BIG;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int key = j0 + 8 * c + i;
-            const float v = (i < 4 ? sacc[0][i] : sacc[1][i - 4]) * sc2;
-            sv[i] = (key >= lo && key <= pos) ? v : LAT_NEG_BIG;
+        for (int i = 0; i < 4; ++i) {
+            const int key = j0 + 16 * wave + 4 * c + i;
+            sv[i] = (key >= lo && key <= pos) ? sacc[i] * sc2 : LAT_NEG_BIG;
             mx = fmaxf(mx, sv[i]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, LLE_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, LLE_WAVE));
+        if (c == 0) s_max[buf][wave][r] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(s_max[buf][0][r], s_max[buf][1][r]), fmaxf(s_max[buf][2][r], s_max[buf][3][r]));
         const float m_new = fmaxf(m, mx);
         const float alpha = exp2f(m - m_new);
-        lbf16x8 pb;
+        lbf16x4 pw;
         float psum = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const float p = sv[i] <= 0.5f * LAT_NEG_BIG ? 0.f : exp2f(sv[i] - m_new);
             psum += p;
-            pb[i] = (bf16_t)p;
+            pw[i] = (bf16_t)p;
         }
         l = l * alpha + psum;
         m = m_new;
-        const int gkey = j0 + 8 * c;  // this lane's eight keys, inside one page
-        const bool gok = gkey + 7 >= lo_min && gkey <= kmax;
-        const bf16_t* vt = pages + (int64_t)(gok ? table[gkey / P] : 0) * page_stride + (int64_t)P * rank + gkey % P;
+        *(lbf16x4*)&s_p[buf][r][16 * wave + 4 * c] = pw;
+        __syncthreads();
+        if (__any(alpha != 1.0f)) {
 #pragma unroll
-        for (int n = 0; n < 2 * RK; ++n) {
-            if (16 * n < rank) {
-                o[n] *= alpha;
-                const lbf16x8 a = gok ? *(const lbf16x8*)(vt + (int64_t)(16 * n + r) * P) : lat_zero8();
-                o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[n], 0, 0, 0);
-            }
+            for (int i = 0; i < NT; ++i) o[i] *= alpha;
+        }
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            const lbf16x8 pb = *(const lbf16x8*)&s_p[buf][r][32 * kk + 8 * c];
+#pragma unroll
+            for (int i = 0; i < NT; ++i)
+                if (!PAD || 16 * (wave * NT + i) < rank)
+                    o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[kk][i], pb, o[i], 0, 0, 0);
         }
     }
     l += __shfl_xor(l, 16, LLE_WAVE);
     l += __shfl_xor(l, 32, LLE_WAVE);
+    if (c == 0) s_l[wave][r] = l;
+    __syncthreads();
+    l = (s_l[0][r] + s_l[1][r]) + (s_l[2][r] + s_l[3][r]);
     if (!valid) return;
     const int64_t grow = (int64_t)(q0 + t) * H + h;
     if (nsplit == 1) {
         const float inv = 1.0f / l;
         bf16_t* orow = out + grow * rank;
 #pragma unroll
-        for (int n = 0; n < 2 * RK; ++n) {
+        for (int i = 0; i < NT; ++i) {
+            const int n = wave * NT + i;
             if (16 * n < rank) {
                 lbf16x4 v;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(o[n][i] * inv);
+                for (int e = 0; e < 4; ++e) v[e] = (bf16_t)(o[i][e] * inv);
                 *(lbf16x4*)(orow + 16 * n + 4 * c) = v;
             }
         }
     } else {
         float* wo = ws_o + (grow * nsplit + split) * rank;
 #pragma unroll
-        for (int n = 0; n < 2 * RK; ++n)
-            if (16 * n < rank) *(lf32x4*)(wo + 16 * n + 4 * c) = o[n];
-        if (c == 0) {
+        for (int i = 0; i < NT; ++i) {
+            const int n = wave * NT + i;
+            if (16 * n < rank) *(lf32x4*)(wo + 16 * n + 4 * c) = o[i];
+        }
+        if (c == 0 && wave == 0) {
             ws_ml[(grow * nsplit + split) * 2] = m;
             ws_ml[(grow * nsplit + split) * 2 + 1] = l;
         }
     }
 }
 
-// one workgroup per (token, head): the ranges' results weighted by 2^(m_i - max m) and normalised
-__global__ __launch_bounds__(128) void latent_combine_kernel(const float* __restrict__ ws_o,
+// grid (rows, ceil(rank / 256)): the ranges' results weighted by 2^(m_i - max m) and normalised, one element a thread
+__global__ __launch_bounds__(256) void latent_combine_kernel(const float* __restrict__ ws_o,
                                                               const float* __restrict__ ws_ml,
                                                               bf16_t* __restrict__ out, int rank, int nsplit) {
+    __shared__ float weight[64];
     const int64_t row = blockIdx.x;
     const float* ml = ws_ml + row * nsplit * 2;
     float M = LAT_NEG_BIG;
     for (int i = 0; i < nsplit; ++i) M = fmaxf(M, ml[2 * i]);
     float L = 0.f;
     for (int i = 0; i < nsplit; ++i) L += ml[2 * i + 1] * exp2f(ml[2 * i] - M);
-    const float inv = 1.0f / L;
-    for (int e = threadIdx.x; e < rank; e += blockDim.x) {
-        float acc = 0.f;
-        for (int i = 0; i < nsplit; ++i) acc += ws_o[(row * nsplit + i) * rank + e] * exp2f(ml[2 * i] - M);
-        out[row * rank + e] = (bf16_t)(acc * inv);
-    }
+    if (threadIdx.x < nsplit) weight[threadIdx.x] = exp2f(ml[2 * threadIdx.x] - M) / L;
+    __syncthreads();
+    const int e = blockIdx.y * blockDim.x + threadIdx.x;
+    if (e >= rank) return;
+    const float* src = ws_o + row * nsplit * rank + e;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int i = 0; i < nsplit; ++i) acc += src[(int64_t)i * rank] * weight[i];
+    out[row * rank + e] = (bf16_t)acc;
 }
 
 // q_lat bfloat16 [N, H, rank] with strides that are multiples of 8; rank a multiple of 16 up to 512, rot a
@@ -424,32 +464,40 @@ extern "C" int lle_latent_attention_mfma(const void* q_lat, int64_t ql_stride_n,
                                          int tiles_max, int nsplit, hipStream_t stream) {
     if (N <= 0 || S <= 0 || H <= 0 || tiles_max <= 0) return 0;
     if (rank <= 0 || rank > 512 || rank % 16 || rot < 0 || rot > 64 || rot % 8 || P <= 0 || P % 16 ||
-        ql_stride_n % 8 || ql_stride_h % 8 || page_stride % 8 || nsplit < 1 || (nsplit > 1 && (!ws_o || !ws_ml)))
+        ql_stride_n % 8 || ql_stride_h % 8 || page_stride % 8 || nsplit < 1 || nsplit > 64 ||
+        (nsplit > 1 && (!ws_o || !ws_ml)))
         return (int)hipErrorInvalidValue;
     const int64_t items = (int64_t)S * tiles_max * nsplit;
     if (items > 0x7fffffff) return (int)hipErrorInvalidValue;
     const int RK = rank <= 64 ? 2 : rank <= 128 ? 4 : rank <= 256 ? 8 : 16;
     const int RR = rot <= 32 ? 1 : 2;
+    const bool pad = rank != 32 * RK || rot != 32 * RR;
 #define LAT_LAUNCH(K, R)                                                                                              \
-    latent_attention_mfma_kernel<K, R><<<(int)items, 64, 0, stream>>>(                                                \
+    if (pad)                                                                                                          \
+        LAT_LAUNCH_(K, R, true);                                                                                      \
+    else                                                                                                              \
+        LAT_LAUNCH_(K, R, false)
+#define LAT_LAUNCH_(K, R, PADDED)                                                                                     \
+    latent_attention_mfma_kernel<K, R, PADDED><<<(int)items, 256, 0, stream>>>(                                        \
         (const bf16_t*)q_lat, ql_stride_n, ql_stride_h, (const float*)q_rot, (const bf16_t*)pages, page_stride, P,    \
         rank, rot, (const int32_t*)block_table, max_pages, (const int32_t*)seq_slots, (const int32_t*)cu_tokens,      \
         (const int32_t*)kv_lens, (const float*)sink, window, scale, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, H,     \
         tiles_max, nsplit)
     if (RR == 1) {
-        if (RK == 2) LAT_LAUNCH(2, 1);
-        else if (RK == 4) LAT_LAUNCH(4, 1);
-        else if (RK == 8) LAT_LAUNCH(8, 1);
-        else LAT_LAUNCH(16, 1);
+        if (RK == 2) { LAT_LAUNCH(2, 1); }
+        else if (RK == 4) { LAT_LAUNCH(4, 1); }
+        else if (RK == 8) { LAT_LAUNCH(8, 1); }
+        else { LAT_LAUNCH(16, 1); }
     } else {
-        if (RK == 2) LAT_LAUNCH(2, 2);
-        else if (RK == 4) LAT_LAUNCH(4, 2);
-        else if (RK == 8) LAT_LAUNCH(8, 2);
-        else LAT_LAUNCH(16, 2);
+        if (RK == 2) { LAT_LAUNCH(2, 2); }
+        else if (RK == 4) { LAT_LAUNCH(4, 2); }
+        else if (RK == 8) { LAT_LAUNCH(8, 2); }
+        else { LAT_LAUNCH(16, 2); }
     }
 #undef LAT_LAUNCH
+#undef LAT_LAUNCH_
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    if (nsplit > 1) latent_combine_kernel<<<N * H, 128, 0, stream>>>((const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, rank, nsplit);
+    if (nsplit > 1) latent_combine_kernel<<<dim3(N * H, (rank + 255) / 256), 256, 0, stream>>>((const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, rank, nsplit);
     LLE_RETURN_LAUNCH_STATUS();
 }

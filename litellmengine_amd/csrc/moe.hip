@@ -64,10 +64,27 @@ extern "C" int lle_moe_route(const void* logits, const void* bias, void* ids, vo
     LLE_RETURN_LAUNCH_STATUS();
 }
 
+typedef bf16_t wbf16x8 __attribute__((ext_vector_type(8)));
+
+// sum over K of a[k] b[k] by one wavefront, every lane gets it; 16-byte loads where the rows allow them
 template <typename T>
 __device__ __forceinline__ float wave_dot(const T* __restrict__ a, const T* __restrict__ b, int K) {
     float acc = 0.f;
-    for (int k = threadIdx.x % LLE_WAVE; k < K; k += LLE_WAVE) acc += to_f32<T>(a[k]) * to_f32<T>(b[k]);
+    const int lane = threadIdx.x % LLE_WAVE;
+    if (sizeof(T) == 2 && K % 8 == 0) {
+        for (int k = lane * 8; k < K; k += LLE_WAVE * 8) {
+            const wbf16x8 av = *(const wbf16x8*)((const bf16_t*)a + k), bv = *(const wbf16x8*)((const bf16_t*)b + k);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc += (float)av[i] * (float)bv[i];
+        }
+    } else if (sizeof(T) == 4 && K % 4 == 0) {
+        for (int k = lane * 4; k < K; k += LLE_WAVE * 4) {
+            const float4 av = *(const float4*)((const float*)a + k), bv = *(const float4*)((const float*)b + k);
+            acc += av.x * bv.x + av.y * bv.y + av.z * bv.z + av.w * bv.w;
+        }
+    } else {
+        for (int k = lane; k < K; k += LLE_WAVE) acc += to_f32<T>(a[k]) * to_f32<T>(b[k]);
+    }
     return wave_sum(acc);
 }
 

@@ -808,6 +808,7 @@ class HipOps:
                           a_ptr, b_ptr, c_ptr, N, O, K, heads * xw, K, heads * O, F32, F32)
         return out
 
+    LATENT_GROUPS_PER_CU = 1
     force_generic_latent = False  # tests flip this to compare the two kernels
     last_latent_kernel = None  # (which kernel, key ranges) of the last latent_attention call: for tests
 
@@ -820,12 +821,12 @@ class HipOps:
         return torch.bfloat16 if mfma else torch.float32
 
     def latent_splits(self, num_seqs: int, heads: int, max_q_len: int, max_kv_len: int, window: int) -> int:
-        """Key ranges per 16-row tile of the matrix-core kernel: enough wavefronts for four on every CU,
-        at least two 32-key steps each, at most 64."""
+        """Key ranges per 16-row tile of the matrix-core kernel: enough workgroups (of four wavefronts) for
+        LATENT_GROUPS_PER_CU on every CU, at least two 64-key steps each, at most 64."""
         tiles = max(1, num_seqs) * -(-max(1, max_q_len) * heads // 16)
         span = min(max_kv_len, window + max_q_len) if window else max_kv_len
-        steps = -(-max(1, span) // 32)
-        return int(max(1, min(-(-4 * self.compute_units() // tiles), steps // 2, 64)))
+        steps = -(-max(1, span) // 64)
+        return int(max(1, min(-(-self.LATENT_GROUPS_PER_CU * self.compute_units() // tiles), steps // 2, 64)))
 
     def latent_attention(self, q_lat, q_rot, pages, page_size: int, rank: int, rot: int, block_table, seq_slots,
                          cu_tokens, kv_lens, token_seq, sink, window: Optional[int], scale: float, max_q_len: int,

@@ -9,8 +9,8 @@
 // The recurrence is linear in S: S_out = A S_in + B with A = prod (1 - z), so the tokens of a
 // long portion are cut into pieces that are scanned side by side:
 //   a short portion (or a decoded token): one thread per (request, channel) walks the tokens;
-//   a long portion: every piece first reduces its (A, B); a second launch starts each piece from the
-//   state that the pieces before it give (a short walk over the pieces' A and B) and walks its tokens.
+//   a long portion: every piece first reduces its (A, B); a short walk over the pieces' (A, B) gives the
+//   state each piece starts from (and the request's new state); then every piece walks its tokens.
 #include "common.h"
 
 LLE_DEFINE_ERROR_STRING()
@@ -31,9 +31,9 @@ __device__ __forceinline__ GruStep gru_gates(const void* zxg, int dtype, int64_t
     return g;
 }
 
-// grid (requests, pieces, channel blocks).  pieces == 1: the whole walk.  pieces > 1 and `pass` 0: only
-// (A, B) of the piece, to part[(s * pieces + piece) * 2 W ...]; `pass` 1: the start state from the
-// pieces before, then the walk; the last piece writes the state back.
+// grid (requests, pieces, channel blocks).  pieces == 1: the whole walk (`pass` 1).  pieces > 1: `pass` 0
+// leaves (A, B) of every piece in part[(s * pieces + piece) * 2 W ...]; mingru_carry_kernel turns them
+// into the state each piece starts from (and writes the request's new state); `pass` 1 walks the tokens.
 template <typename TO>
 __global__ __launch_bounds__(256) void mingru_scan_kernel(const void* __restrict__ zxg, int in_dtype,
                                                            const float* __restrict__ z_bias,
@@ -52,50 +52,48 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(const void* __restrict
     const int t0 = q0 + piece * per;
     const int t1 = min(q1, t0 + per);
     const float bz = z_bias[ch], bx = x_bias[ch];
-    float* st = state + (int64_t)seq_slots[s] * W + ch;
+    float* p = part + ((int64_t)s * pieces + piece) * 2 * W;
     if (pieces > 1 && pass == 0) {
         float A = 1.f, B = 0.f;
+#pragma unroll 4
         for (int t = t0; t < t1; ++t) {
             const GruStep g = gru_gates(zxg, in_dtype, t, W, ch, bz, bx);
             A *= 1.f - g.z;
             B = (1.f - g.z) * B + g.z * g.c;
         }
-        float* p = part + ((int64_t)s * pieces + piece) * 2 * W;
         p[ch] = A;
         p[W + ch] = B;
         return;
     }
-    float S = *st;
-    for (int k = 0; k < piece; ++k) {  // (pieces > 1 only) the pieces before this one, in order
-        const float* p = part + ((int64_t)s * pieces + k) * 2 * W;
-        S = p[ch] * S + p[W + ch];
-    }
+    float* st = state + (int64_t)seq_slots[s] * W + ch;
+    float S = pieces > 1 ? p[ch] : *st;  // (pieces > 1: the carry that mingru_carry_kernel left in A's place)
+#pragma unroll 4
     for (int t = t0; t < t1; ++t) {
         const GruStep g = gru_gates(zxg, in_dtype, t, W, ch, bz, bx);
         S = (1.f - g.z) * S + g.z * g.c;
         const float gate = load_as_f32(zxg, (int64_t)t * 3 * W + 2 * W + ch, in_dtype);
         out[(int64_t)t * W + ch] = from_f32<TO>(S * (gate * sigmoid_f(gate)));
     }
-    if (piece == pieces - 1) {
-        if (pieces > 1) {
-            // every piece has read the old state before anybody writes the new one: the writer is
-            // the last piece, and the others only read `part` and the old state in THIS launch;
-            // so the new state goes to the spare half of the last piece's `part` entry and a
-            // third, tiny launch copies it (see lle_mingru_scan)
-            part[((int64_t)s * pieces + piece) * 2 * W + ch] = S;
-        } else {
-            *st = S;
-        }
-    }
+    if (pieces == 1) *st = S;
 }
 
-__global__ __launch_bounds__(256) void mingru_state_kernel(float* __restrict__ state,
+// one thread per (request, channel): walks the pieces' (A, B) in order, replaces every A by the state its
+// piece starts from, and writes the state after the last piece back to the request's row
+__global__ __launch_bounds__(256) void mingru_carry_kernel(float* __restrict__ state,
                                                             const int32_t* __restrict__ seq_slots,
-                                                            const float* __restrict__ part, int W, int pieces) {
+                                                            float* __restrict__ part, int W, int pieces) {
     const int s = blockIdx.x;
     const int ch = blockIdx.y * blockDim.x + threadIdx.x;
     if (ch >= W) return;
-    state[(int64_t)seq_slots[s] * W + ch] = part[((int64_t)s * pieces + pieces - 1) * 2 * W + ch];
+    float* st = state + (int64_t)seq_slots[s] * W + ch;
+    float S = *st;
+    for (int k = 0; k < pieces; ++k) {
+        float* p = part + ((int64_t)s * pieces + k) * 2 * W;
+        const float A = p[ch], B = p[W + ch];
+        p[ch] = S;
+        S = A * S + B;
+    }
+    *st = S;
 }
 
 // `part`: float32 [S * pieces * 2 W] when pieces > 1 (else unused)
@@ -117,11 +115,14 @@ extern "C" int lle_mingru_scan(const void* zxg, int in_dtype, const void* z_bias
                                                                   (const int32_t*)seq_slots,
                                                                   (const int32_t*)cu_tokens, (bf16_t*)out,
                                                                   (float*)part, W, pieces, pass);
-        const hipError_t e = hipGetLastError();
+        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
+        if (pass == 0) {
+            mingru_carry_kernel<<<dim3(S, (W + 255) / 256), 256, 0, stream>>>((float*)state, (const int32_t*)seq_slots,
+                                                                                (float*)part, W, pieces);
+            e = hipGetLastError();
+            if (e != hipSuccess) return (int)e;
+        }
     }
-    if (pieces > 1)
-        mingru_state_kernel<<<dim3(S, (W + 255) / 256), 256, 0, stream>>>((float*)state, (const int32_t*)seq_slots,
-                                                                            (const float*)part, W, pieces);
-    LLE_RETURN_LAUNCH_STATUS();
+    return 0;
 }
