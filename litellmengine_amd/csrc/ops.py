@@ -736,7 +736,7 @@ class HipOps:
         _need(cu_tokens.shape == (S + 1,), "cu_tokens must be [S + 1]")
         out = torch.empty((N, W), dtype=out_dtype, device=zxg.device)
         pieces = max(1, min(1024, -(-max(1, max_q_len) // self.MINGRU_PIECE)))
-        part = torch.empty((S * pieces * 2 * W,), dtype=torch.float32, device=zxg.device) if pieces > 1 else None
+        part = torch.empty((S * pieces * 3 * W,), dtype=torch.float32, device=zxg.device) if pieces > 1 else None
         self._run("recurrent", "lle_mingru_scan", [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _P],
                   _ptr(zxg), dtype_code(zxg.dtype), _ptr(z_bias), _ptr(x_bias), _ptr(state), _ptr(seq_slots),
                   _ptr(cu_tokens), _ptr(out), dtype_code(out_dtype), _ptr(part), S, W, pieces)

@@ -32,7 +32,7 @@ __device__ __forceinline__ GruStep gru_gates(const void* zxg, int dtype, int64_t
 }
 
 // grid (requests, pieces, channel blocks).  pieces == 1: the whole walk (`pass` 1).  pieces > 1: `pass` 0
-// leaves (A, B) of every piece in part[(s * pieces + piece) * 2 W ...]; mingru_carry_kernel turns them
+// leaves (A, B) of every piece in part[(s * pieces + piece) * 3 W ...]; mingru_carry_kernel turns them
 // into the state each piece starts from (and writes the request's new state); `pass` 1 walks the tokens.
 template <typename TO>
 __global__ __launch_bounds__(256) void mingru_scan_kernel(const void* __restrict__ zxg, int in_dtype,
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(const void* __restrict
     const int t0 = q0 + piece * per;
     const int t1 = min(q1, t0 + per);
     const float bz = z_bias[ch], bx = x_bias[ch];
-    float* p = part + ((int64_t)s * pieces + piece) * 2 * W;
+    float* p = part + ((int64_t)s * pieces + piece) * 3 * W;
     if (pieces > 1 && pass == 0) {
         float A = 1.f, B = 0.f;
 #pragma unroll 4
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(const void* __restrict
         return;
     }
     float* st = state + (int64_t)seq_slots[s] * W + ch;
-    float S = pieces > 1 ? p[ch] : *st;  // (pieces > 1: the carry that mingru_carry_kernel left in A's place)
+    float S = pieces > 1 ? p[2 * W + ch] : *st;  // (pieces > 1: the carry that mingru_carry_kernel left)
 #pragma unroll 4
     for (int t = t0; t < t1; ++t) {
         const GruStep g = gru_gates(zxg, in_dtype, t, W, ch, bz, bx);
@@ -77,26 +77,38 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(const void* __restrict
     if (pieces == 1) *st = S;
 }
 
-// one thread per (request, channel): walks the pieces' (A, B) in order, replaces every A by the state its
-// piece starts from, and writes the state after the last piece back to the request's row
-__global__ __launch_bounds__(256) void mingru_carry_kernel(float* __restrict__ state,
-                                                            const int32_t* __restrict__ seq_slots,
-                                                            float* __restrict__ part, int W, int pieces) {
+// one thread per (request, channel): walks the pieces' (A, B) in order, leaves beside them the state each
+// piece starts from, and writes the state after the last piece back to the request's row.  (A, B) are read
+// eight pieces at a time, so that their loads travel together: nothing written here is read here.
+__global__ __launch_bounds__(64) void mingru_carry_kernel(float* __restrict__ state,
+                                                           const int32_t* __restrict__ seq_slots,
+                                                           float* __restrict__ part, int W, int pieces) {
     const int s = blockIdx.x;
     const int ch = blockIdx.y * blockDim.x + threadIdx.x;
     if (ch >= W) return;
     float* st = state + (int64_t)seq_slots[s] * W + ch;
+    float* base = part + (int64_t)s * pieces * 3 * W + ch;
     float S = *st;
-    for (int k = 0; k < pieces; ++k) {
-        float* p = part + ((int64_t)s * pieces + k) * 2 * W;
-        const float A = p[ch], B = p[W + ch];
-        p[ch] = S;
-        S = A * S + B;
+    for (int k0 = 0; k0 < pieces; k0 += 8) {
+        float A[8], B[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int k = min(k0 + i, pieces - 1);
+            A[i] = __builtin_nontemporal_load(base + (int64_t)k * 3 * W);
+            B[i] = __builtin_nontemporal_load(base + (int64_t)k * 3 * W + W);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (k0 + i < pieces) {
+                base[(int64_t)(k0 + i) * 3 * W + 2 * W] = S;
+                S = A[i] * S + B[i];
+            }
+        }
     }
     *st = S;
 }
 
-// `part`: float32 [S * pieces * 2 W] when pieces > 1 (else unused)
+// `part`: float32 [S * pieces * 3 W] when pieces > 1 (else unused): A, B and the starting state of every piece
 extern "C" int lle_mingru_scan(const void* zxg, int in_dtype, const void* z_bias, const void* x_bias, void* state,
                                const void* seq_slots, const void* cu_tokens, void* out, int out_dtype, void* part,
                                int S, int W, int pieces, hipStream_t stream) {
@@ -118,7 +130,7 @@ extern "C" int lle_mingru_scan(const void* zxg, int in_dtype, const void* z_bias
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
         if (pass == 0) {
-            mingru_carry_kernel<<<dim3(S, (W + 255) / 256), 256, 0, stream>>>((float*)state, (const int32_t*)seq_slots,
+            mingru_carry_kernel<<<dim3(S, (W + 63) / 64), 64, 0, stream>>>((float*)state, (const int32_t*)seq_slots,
                                                                                 (float*)part, W, pieces);
             e = hipGetLastError();
             if (e != hipSuccess) return (int)e;
