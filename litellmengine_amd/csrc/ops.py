@@ -885,7 +885,7 @@ class HipOps:
         _dev(logits, "router logits", torch.float32)
         _dev(bias, "router bias", torch.float32)
         N, E = logits.shape
-        _need(bias.shape == (E,) and 0 < top <= min(E, 16), "a router picks between 1 and 16 of its experts")
+        _need(bias.shape == (E,) and 0 < top <= min(E, 32), "a router picks between 1 and 32 of its experts")
         ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
         gains = torch.empty((N, top), dtype=torch.float32, device=logits.device)
         self._run("moe", "lle_moe_route", [_P, _P, _P, _P, _I, _I, _I, _P], _ptr(logits), _ptr(bias), _ptr(ids),
