@@ -7,7 +7,7 @@
 //
 // Few tokens (decoding), or float32: every (token, choice) pair streams the rows of its expert's
 // weights, a wavefront per output element.  Many bfloat16 tokens (prompt portions, large batches): the
-// pairs are first put in the order of their experts (a counting sort on the device), then tiles of 64
+// pairs are first put in the order of their experts (a counting sort on the device), then tiles of 128
 // pairs of one expert go through the matrix cores against that expert's weights (moe_*_tile kernels),
 // so that an expert's weights are read once per tile and not once per token; the per-pair results
 // are added up per token, in the order of its choices, by a last kernel.
@@ -157,19 +157,20 @@ extern "C" int lle_moe_experts(const void* x, const void* ids, const void* gains
 // ---------------------------------------------------------------------------------------------
 // Many pairs: sorted by expert, then tiles on the matrix cores (bfloat16).
 //   counts[e]            pairs of expert e                                   moe_count_kernel
-//   first[e], tile0[e]   first sorted row / first 64-row tile of expert e    moe_plan_kernel (one workgroup)
+//   first[e], tile0[e]   first sorted row / first 128-row tile of expert e   moe_plan_kernel (one workgroup)
 //   order[row] = pair, place[pair] = row                                     moe_place_kernel
 // The order of an expert's pairs among themselves is whatever the atomics give; no value depends on it.
 // A tile workgroup finds its expert by walking tile0[] (at most 256 experts), and leaves if the step
-// has fewer tiles than the grid (the grid is sized for the worst case, pairs / 64 + experts).
+// has fewer tiles than the grid (the grid is sized for the worst case, pairs / 128 + experts).
 // Products as C^T = W X^T with v_mfma_f32_16x16x32_bf16: lane (c = lane / 16, r = lane % 16) loads 16
 // bytes of row r of a 16-row tile of W (A) and of X (B) and holds outputs n = 4c .. 4c + 3 of row r.
-// A wavefront keeps 64 rows x 64 outputs (gate_up: 64 rows x 32 gate + 32 up); four wavefronts of a
-// workgroup sit side by side along the outputs and share the X rows through the cache.  (Measured at 2048
-// tokens, 64 experts, top 6, 2048 x 1408: the other way round, four wavefronts of 64 rows each against one
-// block of W rows, is 1.6 times slower.)
+// A wavefront keeps 128 rows x 64 outputs (gate_up: 128 rows x 32 gate + 32 up); four wavefronts of a
+// workgroup sit side by side along the outputs and share the X rows, which pass through LDS once for all of
+// them.  (Measured at 2048 tokens, 64 experts, top 6, 2048 x 1408: four wavefronts of 64 rows each against one
+// shared block of W rows are 1.6 times slower than four side by side along the outputs.)
 // ---------------------------------------------------------------------------------------------
-#define MOE_TM 64
+#define MOE_TM 128
+#define MOE_XS 40  // bfloat16 elements between the X rows in LDS: 32 of a step and 16 bytes to spread the banks
 typedef bf16_t mbf16x8 __attribute__((ext_vector_type(8)));
 typedef bf16_t mbf16x4 __attribute__((ext_vector_type(4)));
 typedef float mf32x4 __attribute__((ext_vector_type(4)));
@@ -179,16 +180,24 @@ __global__ __launch_bounds__(256) void moe_zero_kernel(int32_t* __restrict__ p, 
     if (i < n) p[i] = 0;
 }
 
+// (E <= 256.)  A workgroup counts its 256 pairs in LDS first and then adds one number per expert to the global counts.
 __global__ __launch_bounds__(256) void moe_count_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ counts,
-                                                         int pairs) {
+                                                         int pairs, int E) {
+    __shared__ int32_t local[256];
+    local[threadIdx.x] = 0;
+    __syncthreads();
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
-    if (p < pairs) atomicAdd(&counts[ids[p]], 1);
+    if (p < pairs) atomicAdd(&local[ids[p]], 1);
+    __syncthreads();
+    if (threadIdx.x < E && local[threadIdx.x]) atomicAdd(&counts[threadIdx.x], local[threadIdx.x]);
 }
 
 // plan = [counts E | cursor E | first E | tile0 E + 1]
-__global__ __launch_bounds__(64) void moe_plan_kernel(int32_t* __restrict__ plan, int E) {
+__global__ __launch_bounds__(256) void moe_plan_kernel(int32_t* __restrict__ plan, int E) {
+    __shared__ int32_t counts[256];
+    if (threadIdx.x < E) counts[threadIdx.x] = plan[threadIdx.x];
+    __syncthreads();
     if (threadIdx.x != 0) return;
-    int32_t* counts = plan;
     int32_t* first = plan + 2 * E;
     int32_t* tile0 = plan + 3 * E;
     int row = 0, tile = 0;
@@ -201,50 +210,74 @@ __global__ __launch_bounds__(64) void moe_plan_kernel(int32_t* __restrict__ plan
     tile0[E] = tile;
 }
 
+// a workgroup numbers its pairs per expert in LDS, takes one range per expert from the global cursor, and places them
 __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ plan,
                                                          int32_t* __restrict__ order, int32_t* __restrict__ place,
                                                          int pairs, int E) {
+    __shared__ int32_t local[256];
+    local[threadIdx.x] = 0;
+    __syncthreads();
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    int e = 0, mine = 0;
+    if (p < pairs) {
+        e = ids[p];
+        mine = atomicAdd(&local[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x < E && local[threadIdx.x])
+        local[threadIdx.x] = plan[2 * E + threadIdx.x] + atomicAdd(&plan[E + threadIdx.x], local[threadIdx.x]);
+    __syncthreads();
     if (p >= pairs) return;
-    const int e = ids[p];
-    const int row = plan[2 * E + e] + atomicAdd(&plan[E + e], 1);
+    const int row = local[e] + mine;
     order[row] = p;
     place[p] = row;
 }
 
-// eight elements from column k on of four rows each (zeros for a row that does not exist or past the end)
-__device__ __forceinline__ void moe_load4(mbf16x8 (&v)[4], const bf16_t* const (&rows)[4], int k, int K) {
+__device__ __forceinline__ mbf16x8 moe_zero8() {
+    mbf16x8 z;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        mbf16x8 z;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) z[e] = (bf16_t)0.0f;
-        v[i] = (rows[i] && k < K) ? *(const mbf16x8*)(rows[i] + k) : z;
-    }
+    for (int e = 0; e < 8; ++e) z[e] = (bf16_t)0.0f;
+    return z;
 }
 
-__device__ __forceinline__ void moe_mfma16(mf32x4 (&acc)[4][4], const mbf16x8 (&a)[4], const mbf16x8 (&b)[4]) {
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[nt][mt], 0, 0, 0);
+__device__ __forceinline__ mbf16x8 moe_load8(const bf16_t* row, int k, int K) {
+    return (row && k < K) ? *(const mbf16x8*)(row + k) : moe_zero8();
 }
 
-// acc += W rows . X rows over K in steps of 32: the operands of the next step are asked for before the
-// current one is multiplied (two sets of registers take turns)
-__device__ __forceinline__ void moe_tile_product(mf32x4 (&acc)[4][4], const bf16_t* const (&wr)[4],
-                                                 const bf16_t* const (&xr)[4], int c, int K) {
-    mbf16x8 a0[4], b0[4], a1[4], b1[4];
-    moe_load4(a0, wr, 8 * c, K);
-    moe_load4(b0, xr, 8 * c, K);
-    for (int k0 = 0; k0 < K; k0 += 64) {
-        moe_load4(a1, wr, k0 + 32 + 8 * c, K);
-        moe_load4(b1, xr, k0 + 32 + 8 * c, K);
-        moe_mfma16(acc, a0, b0);
-        moe_load4(a0, wr, k0 + 64 + 8 * c, K);
-        moe_load4(b0, xr, k0 + 64 + 8 * c, K);
-        moe_mfma16(acc, a1, b1);  // (zeros past the end)
+// acc[nt][mt] += W rows . X rows over K in steps of 32, for a wavefront's 64 outputs (four 16-row tiles of W,
+// straight from memory: nobody else reads them) against the workgroup's 128 X rows (eight tiles), which all four
+// wavefronts share: every thread brings 32 bytes of them into LDS per step (`xrow`: its two rows, columns
+// 8 (thread % 4) on; nullptr for a row that does not exist).  The operands of the next step are asked for before
+// the current one is multiplied; the LDS buffers take turns, one barrier a step.
+__device__ __forceinline__ void moe_tile_product(mf32x4 (&acc)[4][8], const bf16_t* const (&wr)[4],
+                                                 const bf16_t* const (&xrow)[2], bf16_t (*s_x)[MOE_TM][MOE_XS], int K) {
+    const int lane = threadIdx.x % LLE_WAVE, c = lane / 16, r = lane % 16;
+    const int xr = threadIdx.x / 4, xc = 8 * (threadIdx.x % 4);
+    mbf16x8 a[4], x0, x1;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) a[nt] = moe_load8(wr[nt], 8 * c, K);
+    *(mbf16x8*)&s_x[0][xr][xc] = moe_load8(xrow[0], xc, K);
+    *(mbf16x8*)&s_x[0][xr + 64][xc] = moe_load8(xrow[1], xc, K);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += 32, buf ^= 1) {
+        mbf16x8 an[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) an[nt] = moe_load8(wr[nt], k0 + 32 + 8 * c, K);
+        x0 = moe_load8(xrow[0], k0 + 32 + xc, K);
+        x1 = moe_load8(xrow[1], k0 + 32 + xc, K);
+#pragma unroll
+        for (int mt = 0; mt < 8; ++mt) {
+            const mbf16x8 b = *(const mbf16x8*)&s_x[buf][16 * mt + r][8 * c];
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b, acc[nt][mt], 0, 0, 0);
+        }
+        *(mbf16x8*)&s_x[buf ^ 1][xr][xc] = x0;  // (read last in the step before, which every wavefront has left)
+        *(mbf16x8*)&s_x[buf ^ 1][xr + 64][xc] = x1;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) a[nt] = an[nt];
+        __syncthreads();
     }
 }
 
@@ -280,7 +313,7 @@ __device__ __forceinline__ bool moe_find_tile(const int32_t* __restrict__ plan, 
 }
 
 // act[row, f] = silu(x Wg^T) * (x Wu^T) for the sorted rows; items (tile, block of 128 f), 4 wavefronts of 32 f each
-__global__ __launch_bounds__(256) void moe_gate_up_tile_kernel(const bf16_t* __restrict__ x,
+__global__ __launch_bounds__(256, 2) void moe_gate_up_tile_kernel(const bf16_t* __restrict__ x,
                                                                 const int32_t* __restrict__ plan,
                                                                 const int32_t* __restrict__ order,
                                                                 const bf16_t* __restrict__ gate_up,
@@ -289,15 +322,14 @@ __global__ __launch_bounds__(256) void moe_gate_up_tile_kernel(const bf16_t* __r
     MoeTile t;
     int tile, block;
     if (!moe_grid_item(tiles, blocks, tile, block) || !moe_find_tile(plan, E, tile, t)) return;
+    __shared__ __attribute__((aligned(16))) bf16_t s_x[2][MOE_TM][MOE_XS];
     const int lane = threadIdx.x % LLE_WAVE, c = lane / 16, r = lane % 16;
-    const int f0 = (block * 4 + threadIdx.x / LLE_WAVE) * 32;
-    if (f0 >= F) return;
-    const int wrow = 0;
-    const bf16_t* xr[4];
+    const int f0 = (block * 4 + threadIdx.x / LLE_WAVE) * 32;  // (a wavefront past F multiplies zeros: it shares the barriers)
+    const bf16_t* xrow[2];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-        const int row = wrow + mt * 16 + r;
-        xr[mt] = row < t.rows ? x + (int64_t)(order[t.row0 + row] / top) * K : nullptr;
+    for (int j = 0; j < 2; ++j) {
+        const int row = threadIdx.x / 4 + 64 * j;
+        xrow[j] = row < t.rows ? x + (int64_t)(order[t.row0 + row] / top) * K : nullptr;
     }
     const bf16_t* w = gate_up + (int64_t)t.expert * 2 * F * K;
     const bf16_t* wr[4];  // gate rows f0 + r, f0 + 16 + r, then the up rows of the same f
@@ -306,15 +338,15 @@ __global__ __launch_bounds__(256) void moe_gate_up_tile_kernel(const bf16_t* __r
         const int f = f0 + (nt % 2) * 16 + r;
         wr[nt] = f < F ? w + (int64_t)((nt / 2) * F + f) * K : nullptr;
     }
-    mf32x4 acc[4][4];
+    mf32x4 acc[4][8];
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mf32x4{0.f, 0.f, 0.f, 0.f};
-    moe_tile_product(acc, wr, xr, c, K);
+        for (int mt = 0; mt < 8; ++mt) acc[nt][mt] = mf32x4{0.f, 0.f, 0.f, 0.f};
+    moe_tile_product(acc, wr, xrow, s_x, K);
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-        const int row = wrow + mt * 16 + r;
+    for (int mt = 0; mt < 8; ++mt) {
+        const int row = mt * 16 + r;
         if (row >= t.rows) continue;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -332,22 +364,21 @@ __global__ __launch_bounds__(256) void moe_gate_up_tile_kernel(const bf16_t* __r
 }
 
 // y[row, o] = act[row] Wd[e]^T for the sorted rows, float32; items (tile, block of 256 o), 4 wavefronts of 64 o each
-__global__ __launch_bounds__(256) void moe_down_tile_kernel(const bf16_t* __restrict__ act,
+__global__ __launch_bounds__(256, 2) void moe_down_tile_kernel(const bf16_t* __restrict__ act,
                                                              const int32_t* __restrict__ plan,
                                                              const bf16_t* __restrict__ down, float* __restrict__ y,
                                                              int E, int F, int H, int tiles, int blocks) {
     MoeTile t;
     int tile, block;
     if (!moe_grid_item(tiles, blocks, tile, block) || !moe_find_tile(plan, E, tile, t)) return;
+    __shared__ __attribute__((aligned(16))) bf16_t s_x[2][MOE_TM][MOE_XS];
     const int lane = threadIdx.x % LLE_WAVE, c = lane / 16, r = lane % 16;
-    const int o0 = (block * 4 + threadIdx.x / LLE_WAVE) * 64;
-    if (o0 >= H) return;
-    const int wrow = 0;
-    const bf16_t* xr[4];
+    const int o0 = (block * 4 + threadIdx.x / LLE_WAVE) * 64;  // (a wavefront past H multiplies zeros: it shares the barriers)
+    const bf16_t* xrow[2];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-        const int row = wrow + mt * 16 + r;
-        xr[mt] = row < t.rows ? act + (int64_t)(t.row0 + row) * F : nullptr;
+    for (int j = 0; j < 2; ++j) {
+        const int row = threadIdx.x / 4 + 64 * j;
+        xrow[j] = row < t.rows ? act + (int64_t)(t.row0 + row) * F : nullptr;
     }
     const bf16_t* wr[4];
 #pragma unroll
@@ -355,15 +386,15 @@ __global__ __launch_bounds__(256) void moe_down_tile_kernel(const bf16_t* __rest
         const int o = o0 + nt * 16 + r;
         wr[nt] = o < H ? down + ((int64_t)t.expert * H + o) * F : nullptr;
     }
-    mf32x4 acc[4][4];
+    mf32x4 acc[4][8];
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mf32x4{0.f, 0.f, 0.f, 0.f};
-    moe_tile_product(acc, wr, xr, c, F);
+        for (int mt = 0; mt < 8; ++mt) acc[nt][mt] = mf32x4{0.f, 0.f, 0.f, 0.f};
+    moe_tile_product(acc, wr, xrow, s_x, F);
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-        const int row = wrow + mt * 16 + r;
+    for (int mt = 0; mt < 8; ++mt) {
+        const int row = mt * 16 + r;
         if (row >= t.rows) continue;
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt) {
@@ -401,8 +432,8 @@ extern "C" int lle_moe_experts_tiled(const void* x, const void* ids, const void*
     const int pairs = (int)pairs64;
     const int tiles = pairs / MOE_TM + E;  // at most: every expert leaves one tile partly empty
     moe_zero_kernel<<<(2 * E + 255) / 256, 256, 0, stream>>>((int32_t*)plan, 2 * E);
-    moe_count_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>((const int32_t*)ids, (int32_t*)plan, pairs);
-    moe_plan_kernel<<<1, 64, 0, stream>>>((int32_t*)plan, E);
+    moe_count_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>((const int32_t*)ids, (int32_t*)plan, pairs, E);
+    moe_plan_kernel<<<1, 256, 0, stream>>>((int32_t*)plan, E);
     moe_place_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>((const int32_t*)ids, (int32_t*)plan, (int32_t*)order,
                                                                (int32_t*)place, pairs, E);
     const int fb = (F + 127) / 128, hb = (H + 255) / 256;

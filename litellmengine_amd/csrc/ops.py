@@ -898,7 +898,7 @@ class HipOps:
         """x [N, K]; ids, gains [N, top]; gate_up [E, 2 F, K] (gate rows, then up rows); down [E, H, F] ->
         float32 [N, H]: sum_k gains[n, k] * down[e] (silu(gate[e] x) * (up[e] x)), e = ids[n, k].
         Few pairs, or float32: every pair streams its expert's rows.  Many bfloat16 pairs: sorted by expert
-        on the device, then tiles of 64 pairs of one expert on the matrix cores."""
+        on the device, then tiles of 128 pairs of one expert on the matrix cores."""
         _dev(x, "x")
         _dev(ids, "ids", torch.int32)
         _dev(gains, "gains", torch.float32)
