@@ -238,6 +238,7 @@ extern "C" int lle_latent_attention_generic(const void* q_lat, int q_lat_dtype, 
 // accumulators per wavefront is what leaves registers for that.  With `nsplit` > 1 a tile's keys
 // are cut into ranges whose unnormalised results (and m, l) go to a workspace and are merged by
 // latent_combine_kernel; the sink (m = sink, l = 1) belongs to the first range.
+// RT = row tiles of one workgroup (1 or 2): with two, the step's operands serve 32 rows.
 // RK = 32-element steps over the latent (rank <= 32 RK, padded with zeros), RR the same for k_rot.
 // PAD: rank < 32 RK or rot < 32 RR, and the operands' tails are filled with zeros under a condition.
 // Without it every load is unconditional (a key outside the tile's range is read from the nearest one
@@ -258,7 +259,7 @@ __device__ __forceinline__ lbf16x8 lat_zero8() {
     return z;
 }
 
-template <int RK, int RR, bool PAD>
+template <int RK, int RR, bool PAD, int RT>
 __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ q_lat, int64_t ql_stride_n, int64_t ql_stride_h, const float* __restrict__ q_rot,
     const bf16_t* __restrict__ pages, int64_t page_stride, int P, int rank, int rot,
@@ -267,10 +268,10 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     int window, float scale, bf16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml, int H,
     int tiles_max, int nsplit) {
     constexpr int NT = RK / 2;  // value tiles (16 latent elements each) of one wavefront, of 2 RK
-    __shared__ float s_max[2][4][16];
-    __shared__ __attribute__((aligned(16))) bf16_t s_p[2][16][LAT_P_STRIDE];
-    __shared__ float s_l[4][16];
-    __shared__ __attribute__((aligned(16))) bf16_t s_q[16][32 * (RK + RR) + 8];  // (8 more: rows 16 bytes off the banks)
+    __shared__ float s_max[2][RT][4][16];
+    __shared__ __attribute__((aligned(16))) bf16_t s_p[2][RT][16][LAT_P_STRIDE];
+    __shared__ float s_l[RT][4][16];
+    __shared__ __attribute__((aligned(16))) bf16_t s_q[RT][16][32 * (RK + RR) + 8];  // (8 more: rows 16 bytes off the banks)
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE, c = lane / 16, r = lane % 16;
     int item = blockIdx.x;
     const int split = item % nsplit;
@@ -279,45 +280,57 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const int tile = tiles_max - 1 - item % tiles_max, s = item / tiles_max;
     const int q0 = cu_tokens[s], q_len = cu_tokens[s + 1] - q0;
     const int rows = q_len * H;
-    if (tile * 16 >= rows) return;  // (the whole workgroup)
+    const int row0 = tile * 16 * RT;  // the workgroup's RT tiles of 16 rows: row0 .. row0 + 16 RT - 1
+    if (row0 >= rows) return;  // (the whole workgroup)
     const int past = kv_lens[s] - q_len;
-    const int rho = tile * 16 + r;
-    const bool valid = rho < rows;
-    const int t = valid ? rho / H : 0, h = valid ? rho % H : 0;
-    const int pos = valid ? past + t : -1;  // a row that does not exist sees nothing
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int t_first = (tile * 16) / H, t_last = min(q_len - 1, (tile * 16 + 15) / H);
-    const int kmax = past + t_last;  // the tile's keys: lo_min .. kmax
+    bool valid[RT];
+    int tok[RT], head[RT], pos[RT], lo[RT];
+#pragma unroll
+    for (int u = 0; u < RT; ++u) {
+        const int rho = row0 + 16 * u + r;
+        valid[u] = rho < rows;
+        tok[u] = valid[u] ? rho / H : 0;
+        head[u] = valid[u] ? rho % H : 0;
+        pos[u] = valid[u] ? past + tok[u] : -1;  // a row that does not exist sees nothing
+        lo[u] = window > 0 ? max(0, pos[u] - window + 1) : 0;
+    }
+    const int t_first = row0 / H, t_last = min(q_len - 1, (row0 + 16 * RT - 1) / H);
+    const int kmax = past + t_last;  // the workgroup's keys: lo_min .. kmax
     const int lo_min = window > 0 ? max(0, past + t_first - window + 1) : 0;
     const int32_t* table = block_table + (int64_t)seq_slots[s] * max_pages;
 
-    // the tile's queries wait in LDS as the B operands of the first product: row r, elements 32 i + 8 c .. + 7
+    // the tiles' queries wait in LDS as the B operands of the first product: row r, elements 32 i + 8 c .. + 7
     // for lane (c, r) and step i; every wavefront writes a quarter of the steps and reads them all
-    {
-        const bf16_t* ql = q_lat + (int64_t)(q0 + t) * ql_stride_n + (int64_t)h * ql_stride_h;
-        const float* qr = q_rot + ((int64_t)(q0 + t) * H + h) * rot;
+#pragma unroll
+    for (int u = 0; u < RT; ++u) {
+        const bf16_t* ql = q_lat + (int64_t)(q0 + tok[u]) * ql_stride_n + (int64_t)head[u] * ql_stride_h;
+        const float* qr = q_rot + ((int64_t)(q0 + tok[u]) * H + head[u]) * rot;
         for (int i = wave; i < RK + RR; i += 4) {
             lbf16x8 v = lat_zero8();
             if (i < RK) {
                 const int e0 = 32 * i + 8 * c;
-                if (valid && e0 < rank) v = *(const lbf16x8*)(ql + e0);
+                if (valid[u] && e0 < rank) v = *(const lbf16x8*)(ql + e0);
             } else {
                 const int e0 = 32 * (i - RK) + 8 * c;
-                if (valid && e0 < rot) {
+                if (valid[u] && e0 < rot) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) v[e] = (bf16_t)qr[e0 + e];
                 }
             }
-            *(lbf16x8*)&s_q[r][32 * i + 8 * c] = v;
+            *(lbf16x8*)&s_q[u][r][32 * i + 8 * c] = v;
         }
     }
     __syncthreads();
-    lf32x4 o[NT];
+    lf32x4 o[RT][NT];
+    float m[RT], l[RT];
 #pragma unroll
-    for (int i = 0; i < NT; ++i) o[i] = lf32x4{0.f, 0.f, 0.f, 0.f};
-    const bool first = split == 0 && valid;
-    float m = first ? sink[h] * LAT_LOG2E : LAT_NEG_BIG;     // base 2; the same in the row's lanes of every wavefront
-    float l = (first && c == 0 && wave == 0) ? 1.0f : 0.0f;  // this lane's share of the row's sum
+    for (int u = 0; u < RT; ++u) {
+#pragma unroll
+        for (int i = 0; i < NT; ++i) o[u][i] = lf32x4{0.f, 0.f, 0.f, 0.f};
+        const bool first = split == 0 && valid[u];
+        m[u] = first ? sink[head[u]] * LAT_LOG2E : LAT_NEG_BIG;     // base 2; the same in the row's lanes of every wavefront
+        l[u] = (first && c == 0 && wave == 0) ? 1.0f : 0.0f;        // this lane's share of the row's sum
+    }
     const float sc2 = scale * LAT_LOG2E;
 
     const int s_begin = lo_min / LAT_STEP, s_end = kmax / LAT_STEP + 1;
@@ -326,7 +339,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     int buf = 0;
     for (int st = st_lo; st < st_hi; ++st, buf ^= 1) {
         const int j0 = st * LAT_STEP;
-        // every operand of the step is asked for here
+        // every operand of the step is asked for here, once for all the workgroup's row tiles
         lbf16x8 ka[RK + RR];
         {
             const int key = min(max(j0 + 16 * wave + r, lo_min), kmax);  // (outside: masked below)
@@ -353,80 +366,98 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
                 va[kk][i] = (!PAD || 16 * n < rank) ? *(const lbf16x8*)(vt + (int64_t)(16 * n + r) * P) : lat_zero8();
             }
         }
-        lf32x4 sacc = lf32x4{0.f, 0.f, 0.f, 0.f};
+        float sv[RT][4];
 #pragma unroll
-        for (int i = 0; i < RK + RR; ++i)
-            sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[i], *(const lbf16x8*)&s_q[r][32 * i + 8 * c], sacc, 0, 0, 0);
-        float sv[4];
-        float mx = LAT_NEG_BIG;
+        for (int u = 0; u < RT; ++u) {
+            lf32x4 sacc = lf32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = j0 + 16 * wave + 4 * c + i;
-            sv[i] = (key >= lo && key <= pos) ? sacc[i] * sc2 : LAT_NEG_BIG;
-            mx = fmaxf(mx, sv[i]);
+            for (int i = 0; i < RK + RR; ++i)
+                sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[i], *(const lbf16x8*)&s_q[u][r][32 * i + 8 * c], sacc, 0,
+                                                               0, 0);
+            float mx = LAT_NEG_BIG;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = j0 + 16 * wave + 4 * c + i;
+                sv[u][i] = (key >= lo[u] && key <= pos[u]) ? sacc[i] * sc2 : LAT_NEG_BIG;
+                mx = fmaxf(mx, sv[u][i]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, LLE_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, LLE_WAVE));
+            if (c == 0) s_max[buf][u][wave][r] = mx;
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, LLE_WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, LLE_WAVE));
-        if (c == 0) s_max[buf][wave][r] = mx;
         __syncthreads();
-        mx = fmaxf(fmaxf(s_max[buf][0][r], s_max[buf][1][r]), fmaxf(s_max[buf][2][r], s_max[buf][3][r]));
-        const float m_new = fmaxf(m, mx);
-        const float alpha = exp2f(m - m_new);
-        lbf16x4 pw;
-        float psum = 0.f;
+        float alpha[RT];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float p = sv[i] <= 0.5f * LAT_NEG_BIG ? 0.f : exp2f(sv[i] - m_new);
-            psum += p;
-            pw[i] = (bf16_t)p;
+        for (int u = 0; u < RT; ++u) {
+            const float mx = fmaxf(fmaxf(s_max[buf][u][0][r], s_max[buf][u][1][r]),
+                                   fmaxf(s_max[buf][u][2][r], s_max[buf][u][3][r]));
+            const float m_new = fmaxf(m[u], mx);
+            alpha[u] = exp2f(m[u] - m_new);
+            lbf16x4 pw;
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float p = sv[u][i] <= 0.5f * LAT_NEG_BIG ? 0.f : exp2f(sv[u][i] - m_new);
+                psum += p;
+                pw[i] = (bf16_t)p;
+            }
+            l[u] = l[u] * alpha[u] + psum;
+            m[u] = m_new;
+            *(lbf16x4*)&s_p[buf][u][r][16 * wave + 4 * c] = pw;
         }
-        l = l * alpha + psum;
-        m = m_new;
-        *(lbf16x4*)&s_p[buf][r][16 * wave + 4 * c] = pw;
         __syncthreads();
-        if (__any(alpha != 1.0f)) {
 #pragma unroll
-            for (int i = 0; i < NT; ++i) o[i] *= alpha;
-        }
+        for (int u = 0; u < RT; ++u) {
+            if (__any(alpha[u] != 1.0f)) {
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            const lbf16x8 pb = *(const lbf16x8*)&s_p[buf][r][32 * kk + 8 * c];
+                for (int i = 0; i < NT; ++i) o[u][i] *= alpha[u];
+            }
 #pragma unroll
-            for (int i = 0; i < NT; ++i)
-                if (!PAD || 16 * (wave * NT + i) < rank)
-                    o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[kk][i], pb, o[i], 0, 0, 0);
-        }
-    }
-    l += __shfl_xor(l, 16, LLE_WAVE);
-    l += __shfl_xor(l, 32, LLE_WAVE);
-    if (c == 0) s_l[wave][r] = l;
-    __syncthreads();
-    l = (s_l[0][r] + s_l[1][r]) + (s_l[2][r] + s_l[3][r]);
-    if (!valid) return;
-    const int64_t grow = (int64_t)(q0 + t) * H + h;
-    if (nsplit == 1) {
-        const float inv = 1.0f / l;
-        bf16_t* orow = out + grow * rank;
+            for (int kk = 0; kk < 2; ++kk) {
+                const lbf16x8 pb = *(const lbf16x8*)&s_p[buf][u][r][32 * kk + 8 * c];
 #pragma unroll
-        for (int i = 0; i < NT; ++i) {
-            const int n = wave * NT + i;
-            if (16 * n < rank) {
-                lbf16x4 v;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = (bf16_t)(o[i][e] * inv);
-                *(lbf16x4*)(orow + 16 * n + 4 * c) = v;
+                for (int i = 0; i < NT; ++i)
+                    if (!PAD || 16 * (wave * NT + i) < rank)
+                        o[u][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[kk][i], pb, o[u][i], 0, 0, 0);
             }
         }
-    } else {
-        float* wo = ws_o + (grow * nsplit + split) * rank;
+    }
 #pragma unroll
-        for (int i = 0; i < NT; ++i) {
-            const int n = wave * NT + i;
-            if (16 * n < rank) *(lf32x4*)(wo + 16 * n + 4 * c) = o[i];
-        }
-        if (c == 0 && wave == 0) {
-            ws_ml[(grow * nsplit + split) * 2] = m;
-            ws_ml[(grow * nsplit + split) * 2 + 1] = l;
+    for (int u = 0; u < RT; ++u) {
+        l[u] += __shfl_xor(l[u], 16, LLE_WAVE);
+        l[u] += __shfl_xor(l[u], 32, LLE_WAVE);
+        if (c == 0) s_l[u][wave][r] = l[u];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < RT; ++u) {
+        if (!valid[u]) continue;
+        const float lsum = (s_l[u][0][r] + s_l[u][1][r]) + (s_l[u][2][r] + s_l[u][3][r]);
+        const int64_t grow = (int64_t)(q0 + tok[u]) * H + head[u];
+        if (nsplit == 1) {
+            const float inv = 1.0f / lsum;
+            bf16_t* orow = out + grow * rank;
+#pragma unroll
+            for (int i = 0; i < NT; ++i) {
+                const int n = wave * NT + i;
+                if (16 * n < rank) {
+                    lbf16x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = (bf16_t)(o[u][i][e] * inv);
+                    *(lbf16x4*)(orow + 16 * n + 4 * c) = v;
+                }
+            }
+        } else {
+            float* wo = ws_o + (grow * nsplit + split) * rank;
+#pragma unroll
+            for (int i = 0; i < NT; ++i) {
+                const int n = wave * NT + i;
+                if (16 * n < rank) *(lf32x4*)(wo + 16 * n + 4 * c) = o[u][i];
+            }
+            if (c == 0 && wave == 0) {
+                ws_ml[(grow * nsplit + split) * 2] = m[u];
+                ws_ml[(grow * nsplit + split) * 2 + 1] = lsum;
+            }
         }
     }
 }
@@ -454,14 +485,14 @@ __global__ __launch_bounds__(256) void latent_combine_kernel(const float* __rest
 }
 
 // q_lat bfloat16 [N, H, rank] with strides that are multiples of 8; rank a multiple of 16 up to 512, rot a
-// multiple of 8 up to 64, P a multiple of 16.  `tiles_max` = ceil(max_q_len * H / 16).  nsplit > 1 needs
+// multiple of 8 up to 64, P a multiple of 16.  `tiles_max` = ceil(max_q_len * H / (16 row_tiles)).  nsplit > 1 needs
 // ws_o float32 [N H nsplit rank] and ws_ml float32 [N H nsplit 2].
 extern "C" int lle_latent_attention_mfma(const void* q_lat, int64_t ql_stride_n, int64_t ql_stride_h,
                                          const void* q_rot, const void* pages, int64_t page_stride, int P, int rank,
                                          int rot, const void* block_table, int max_pages, const void* seq_slots,
                                          const void* cu_tokens, const void* kv_lens, const void* sink, int window,
                                          float scale, void* out, void* ws_o, void* ws_ml, int N, int S, int H,
-                                         int tiles_max, int nsplit, hipStream_t stream) {
+                                         int tiles_max, int nsplit, int row_tiles, hipStream_t stream) {
     if (N <= 0 || S <= 0 || H <= 0 || tiles_max <= 0) return 0;
     if (rank <= 0 || rank > 512 || rank % 16 || rot < 0 || rot > 64 || rot % 8 || P <= 0 || P % 16 ||
         ql_stride_n % 8 || ql_stride_h % 8 || page_stride % 8 || nsplit < 1 || nsplit > 64 ||
@@ -472,13 +503,18 @@ extern "C" int lle_latent_attention_mfma(const void* q_lat, int64_t ql_stride_n,
     const int RK = rank <= 64 ? 2 : rank <= 128 ? 4 : rank <= 256 ? 8 : 16;
     const int RR = rot <= 32 ? 1 : 2;
     const bool pad = rank != 32 * RK || rot != 32 * RR;
+    if (row_tiles != 1 && row_tiles != 2) return (int)hipErrorInvalidValue;
 #define LAT_LAUNCH(K, R)                                                                                              \
-    if (pad)                                                                                                          \
-        LAT_LAUNCH_(K, R, true);                                                                                      \
+    if (pad && row_tiles == 1)                                                                                        \
+        LAT_LAUNCH_(K, R, true, 1);                                                                                   \
+    else if (pad)                                                                                                     \
+        LAT_LAUNCH_(K, R, true, 2);                                                                                   \
+    else if (row_tiles == 1)                                                                                          \
+        LAT_LAUNCH_(K, R, false, 1);                                                                                  \
     else                                                                                                              \
-        LAT_LAUNCH_(K, R, false)
-#define LAT_LAUNCH_(K, R, PADDED)                                                                                     \
-    latent_attention_mfma_kernel<K, R, PADDED><<<(int)items, 256, 0, stream>>>(                                        \
+        LAT_LAUNCH_(K, R, false, 2)
+#define LAT_LAUNCH_(K, R, PADDED, TILES)                                                                              \
+    latent_attention_mfma_kernel<K, R, PADDED, TILES><<<(int)items, 256, 0, stream>>>(                                \
         (const bf16_t*)q_lat, ql_stride_n, ql_stride_h, (const float*)q_rot, (const bf16_t*)pages, page_stride, P,    \
         rank, rot, (const int32_t*)block_table, max_pages, (const int32_t*)seq_slots, (const int32_t*)cu_tokens,      \
         (const int32_t*)kv_lens, (const float*)sink, window, scale, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, H,     \

@@ -820,10 +820,18 @@ class HipOps:
                 and page_size % 16 == 0 and not self.force_generic_latent)
         return torch.bfloat16 if mfma else torch.float32
 
+    def latent_row_tiles(self, heads: int, max_q_len: int) -> int:
+        """16-row tiles per workgroup of the matrix-core kernel: two for prompt portions (a step's operands then
+        serve 32 rows: measured at rank 512, 2048 tokens, 388 -> 325 us at 16 heads and 758 -> 629 us at 32), one for
+        decoded tokens (two cost a wavefront a SIMD and 2 us of 22 at 32 heads)."""
+        return self.force_latent_row_tiles or (2 if max_q_len >= 4 and max_q_len * heads >= 64 else 1)
+
+    force_latent_row_tiles = 0  # tests set 1 or 2
+
     def latent_splits(self, num_seqs: int, heads: int, max_q_len: int, max_kv_len: int, window: int) -> int:
         """Key ranges per 16-row tile of the matrix-core kernel: enough workgroups (of four wavefronts) for
         LATENT_GROUPS_PER_CU on every CU, at least two 64-key steps each, at most 64."""
-        tiles = max(1, num_seqs) * -(-max(1, max_q_len) * heads // 16)
+        tiles = max(1, num_seqs) * -(-max(1, max_q_len) * heads // (16 * self.latent_row_tiles(heads, max_q_len)))
         span = min(max_kv_len, window + max_q_len) if window else max_kv_len
         steps = -(-max(1, span) // 64)
         return int(max(1, min(-(-self.LATENT_GROUPS_PER_CU * self.compute_units() // tiles), steps // 2, 64)))
@@ -856,18 +864,19 @@ class HipOps:
                 and q_lat.stride(0) % 8 == 0 and q_lat.stride(1) % 8 == 0 and pages.stride(0) % 8 == 0
                 and max_q_len > 0 and max_kv_len > 0):
             ns = self.latent_splits(S, H, max_q_len, max_kv_len, win)
+            rt = self.latent_row_tiles(H, max_q_len)
             self.last_latent_kernel = ("matrix cores", ns)
             ws_o = ws_ml = None
             if ns > 1:
                 ws_o = torch.empty((N * H * ns * rank,), dtype=torch.float32, device=pages.device)
                 ws_ml = torch.empty((N * H * ns * 2,), dtype=torch.float32, device=pages.device)
             self._run("latent", "lle_latent_attention_mfma",
-                      [_P, _L, _L, _P, _P, _L, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _F, _P, _P, _P, _I, _I, _I, _I, _I,
+                      [_P, _L, _L, _P, _P, _L, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _F, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                        _P],
                       _ptr(q_lat), q_lat.stride(0), q_lat.stride(1), _ptr(q_rot), _ptr(pages), pages.stride(0),
                       int(page_size), rank, rot, _ptr(block_table), block_table.shape[1], _ptr(seq_slots),
                       _ptr(cu_tokens), _ptr(kv_lens), _ptr(sink), win, float(scale), _ptr(out), _ptr(ws_o), _ptr(ws_ml),
-                      N, S, H, -(-max_q_len * H // 16), ns)
+                      N, S, H, -(-max_q_len * H // (16 * rt)), ns, rt)
             return out
         self.last_latent_kernel = ("generic", 1)
         self._run("latent", "lle_latent_attention_generic",

@@ -155,13 +155,18 @@ def test_latent_attention(dtype, P, rank, rot, H, lens, pasts, window):
         q_lat = rnd((H, N, rank), q_dtype, 24, 0.3).transpose(0, 1)
         args = (q_lat, q_rot, c["pages"], P, rank, rot, c["table"], c["seq_slots"], c["cu"], c["kv_lens"], c["token_seq"],
                 sink, window, 0.11, max(lens), max(c["kv_lens"].tolist()), dtype)
-        got = o.latent_attention(*args)
-        on_cores = q_dtype == torch.bfloat16 and rank % 16 == 0 and rank <= 512 and rot % 8 == 0 and P % 16 == 0
-        assert o.last_latent_kernel[0] == ("matrix cores" if on_cores else "generic")
-        if on_cores and max(pasts) > 1000:
-            assert o.last_latent_kernel[1] > 1  # key ranges, merged
         want = REF.latent_attention(*args)
-        assert got.shape == (N, H, rank) and (got.double() - want.double()).abs().max() < tol(dtype, 2)
+        on_cores = q_dtype == torch.bfloat16 and rank % 16 == 0 and rank <= 512 and rot % 8 == 0 and P % 16 == 0
+        for row_tiles in ((0, 1, 2) if on_cores else (0,)):  # as the sizes choose; one and two 16-row tiles a workgroup
+            o.force_latent_row_tiles = row_tiles
+            try:
+                got = o.latent_attention(*args)
+            finally:
+                o.force_latent_row_tiles = 0
+            assert o.last_latent_kernel[0] == ("matrix cores" if on_cores else "generic")
+            if on_cores and max(pasts) > 1000:
+                assert o.last_latent_kernel[1] > 1  # key ranges, merged
+            assert got.shape == (N, H, rank) and (got.double() - want.double()).abs().max() < tol(dtype, 2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES + ["bfloat16 queries"])
