@@ -49,6 +49,44 @@ def test_trace_gpu(tmp_path, which, dtype):
     print(f"trace {which} {dtype}: worst relative error {worst:.3g}, pool {tb.max_tokens} tokens")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_one_layer_at_a_time_follows_the_plain_model_gpu(tmp_path, which, dtype):
+    """The residual stream after every block: a whole prompt, then the same prompt in two portions and three
+    single tokens through the cache and the state rows (so the first layer that goes wrong is named)."""
+    from litellmengine_amd.cache import CacheManager
+    from litellmengine_amd.engine import ModelRunner, StepEntry
+    from litellmengine_amd.models import load_model
+
+    d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
+    sharpen(d, fixed_routes=dtype == "bfloat16")
+    cfg, w = plain.read_model_dir(d)
+    tokens = random_tokens(70, cfg["vocab"], 3)
+    want = plain.residual_streams(tokens, w, cfg)
+    model = load_model(d, dtype)
+    cache = CacheManager(model, page_size=PAGE_SIZES[which], num_pages=40, max_requests=2, dtype=model.ctx.dtype,
+                         device=model.ctx.device)
+    runner = ModelRunner(model, cache, use_graphs=False)
+    seen = []
+    for b in model.blocks:
+        def wrapped(hidden, delta, step, layer_cache, next_norm=None, inner=b.forward):
+            out = inner(hidden, delta, step, layer_cache, next_norm=next_norm)
+            seen.append(hidden.double().cpu())
+            return out
+        b.forward = wrapped
+    tol = 2e-5 if dtype == "float32" else 4e-2
+    for cuts in ([70], [40, 27, 1, 1, 1]):
+        slot, at = runner.admit(), 0
+        for n in cuts:
+            seen.clear()
+            runner.step([StepEntry(slot, tokens[at : at + n], [])])
+            for i, (got, ref) in enumerate(zip(seen, want)):
+                err = (got - ref[at : at + n]).abs().max() / ref.abs().max()
+                assert err < tol, f"layer {i} ({cfg['layers'][i]['type']}), tokens {at}..{at + n}: {float(err):.3g}"
+            at += n
+        runner.release(slot)
+
+
 # Larger scores carry the rounding of queries and latents further into the softmax weights, and
 # sharper gates carry the rounding of their inputs into the states: the tolerances grow with the factors.
 # (B's scores grow faster with the factor: more elements per head and a larger scale)
