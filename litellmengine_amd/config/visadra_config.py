@@ -69,7 +69,7 @@ def _positive(value: int, what: str) -> int:
 def _mixer_from(kind: str, m: Dict[str, Any], where: str):
     if kind in MINGRU_TYPES:
         return MinGRUSizes(_positive(_required(m, "width", int), f"{where}.mixer.width"))
-    rot = _section(m, "rot", f"{where}.mixer")
+    rot = m.get("rot") if isinstance(m.get("rot"), dict) else {}
     rot_dim = _positive(_required(m, "rot_dim", int), f"{where}.mixer.rot_dim")
     rot_dims = _optional(rot, "dims", int, rot_dim)
     if rot_dims % 2 or not 0 <= rot_dims <= rot_dim:
@@ -83,13 +83,15 @@ def _mixer_from(kind: str, m: Dict[str, Any], where: str):
         rot_dim=rot_dim,
         vdim=_positive(_required(m, "vdim", int), f"{where}.mixer.vdim"),
         kv_rank=_positive(_required(m, "kv_rank", int), f"{where}.mixer.kv_rank"),
-        scale=_required(m, "scale", float),
-        rot_base=_required(rot, "base", float),
+        scale=_optional(m, "scale", float, 0.0),
+        rot_base=_optional(rot, "base", float, 10000.0),
         rot_dims=rot_dims,
         window=window,
     )
     if not sizes.rot_base > 0.0:
         raise ConfigError(f"{where}.mixer.rot.base must be positive")
+    if "scale" not in m or m["scale"] is None:  # the usual one: over all query/key elements of a head
+        sizes = dataclasses.replace(sizes, scale=float(sizes.dim + sizes.rot_dim) ** -0.5)
     return sizes
 
 

@@ -128,6 +128,18 @@ def test_config_round_trip_and_registry(tmp_path, which):
     assert len(model.blocks) == len(CONFIGS[which]["layers"]) and model.vocab_size == cfg.vocab
 
 
+def test_config_defaults():
+    """Without `scale` a head's scores are scaled by 1 / sqrt(dim + rot_dim); without `rot` the base is 10000 and
+    every rotated element turns; without `embedding` and `logit_scale` nothing is scaled."""
+    d = json.loads(json.dumps(CONFIGS["A"]))
+    m = d["layers"][0]["mixer"]
+    del m["scale"], m["rot"], d["embedding"], d["logit_scale"]
+    cfg = VisadraConfig.from_dict(d)
+    a = cfg.layers[0].mixer
+    assert a.scale == (a.dim + a.rot_dim) ** -0.5 and a.rot_base == 10000.0 and a.rot_dims == a.rot_dim
+    assert cfg.embedding_scale == 1.0 and cfg.logit_scale == 1.0
+
+
 def test_config_faults_are_named():
     bad = json.loads(json.dumps(CONFIGS["A"]))
     bad["layers"][1]["type"] = "lstm"
