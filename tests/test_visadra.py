@@ -200,6 +200,8 @@ def test_one_layer_at_a_time_follows_the_plain_model(tmp_path, which):
     runner.step([StepEntry(runner.admit(), tokens, [])])
     for i, (got, ref) in enumerate(zip(seen, want)):
         assert (got - ref).abs().max() < 1e-5, f"layer {i} ({cfg['layers'][i]['type']})"
+    for b in model.blocks:
+        del b.forward  # (the wrappers hold the model in a cycle)
 
 
 def all_ways_trace(requests):

@@ -85,6 +85,8 @@ def test_one_layer_at_a_time_follows_the_plain_model_gpu(tmp_path, which, dtype)
                 assert err < tol, f"layer {i} ({cfg['layers'][i]['type']}), tokens {at}..{at + n}: {float(err):.3g}"
             at += n
         runner.release(slot)
+    for b in model.blocks:
+        del b.forward  # (the wrappers hold the model in a cycle)
 
 
 # Larger scores carry the rounding of queries and latents further into the softmax weights, and

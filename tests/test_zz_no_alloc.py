@@ -26,6 +26,9 @@ def entry_points():
 def test_static_argmax_equals_workspace_argmax_twice_in_a_row():
     from litellmengine_amd.csrc.ops import default_ops
 
+    import gc
+
+    gc.collect()  # what earlier tests left in reference cycles is freed now, not in the middle of a measurement
     ops = default_ops()
     lib, static = entry_points()
     dev = torch.device("cuda", torch.cuda.current_device())
