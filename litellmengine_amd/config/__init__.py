@@ -1,5 +1,6 @@
 from .model_config import ConfigError, Qwen3Config, read_config_json, FULL_ATTENTION, SLIDING_ATTENTION
 from .visadra_config import VisadraConfig
+from .kezasun_config import KezasunConfig
 from .registry import (
     Architecture,
     architecture_of,
@@ -14,6 +15,7 @@ __all__ = [
     "ConfigError",
     "Qwen3Config",
     "VisadraConfig",
+    "KezasunConfig",
     "FULL_ATTENTION",
     "SLIDING_ATTENTION",
     "architecture_of",

@@ -63,7 +63,17 @@ def architecture_of_model_dir(model_dir: str) -> Architecture:
 def load_config(model_dir: str):
     """config.json of a model folder -> the typed configuration of its architecture."""
     d = read_config_json(model_dir)
-    return architecture_of(d).config_class.from_dict(d)
+    config = architecture_of(d).config_class.from_dict(d)
+    if hasattr(config, "with_tensor_shapes"):  # sizes that config.json leaves to the checkpoint's shapes
+        from ..weights.loader import WeightError, checkpoint_header
+
+        try:
+            header = checkpoint_header(model_dir)
+        except WeightError:
+            header = None  # a folder without weights (random-weights mode): the config must say every size itself
+        if header is not None:
+            config = config.with_tensor_shapes({name: shape for name, (_, shape, _) in header.items()})
+    return config
 
 
 def _ensure_builtin() -> None:

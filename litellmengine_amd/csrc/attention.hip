@@ -43,7 +43,8 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void paged_attention_generic_k
     const T* __restrict__ q, const T* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, const int32_t* __restrict__ token_seq, T* __restrict__ out, int nq,
-    int nkv, int d, int page_size, int64_t page_stride, int max_pages, int window, float scale) {
+    int nkv, int d, int page_size, int64_t page_stride, int max_pages, int window, float scale,
+    const float* __restrict__ sinks) {
     __shared__ float s_m[ATT_WAVES], s_l[ATT_WAVES];
     __shared__ float s_acc[ATT_WAVES][ATT_MAX_R * LLE_WAVE];
 
@@ -153,8 +154,10 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void paged_attention_generic_k
     __syncthreads();
     float big = s_m[0];
     for (int w = 1; w < ATT_WAVES; ++w) big = fmaxf(big, s_m[w]);
+    // a sink: one more place in the softmax's sum, with a score of its own and no value
+    const float sink_share = sinks ? expf(sinks[h] - big) : 0.f;
     for (int e = threadIdx.x; e < d; e += blockDim.x) {
-        float num = 0.f, den = 0.f;
+        float num = 0.f, den = sink_share;
         for (int w = 0; w < ATT_WAVES; ++w) {
             const float f = expf(s_m[w] - big);  // a wavefront without keys has l = 0, acc = 0
             num += s_acc[w][e] * f;
@@ -168,7 +171,7 @@ extern "C" int lle_paged_attention_generic(const void* q, const void* kv_layer, 
                                            const void* seq_slots, const void* cu_tokens, const void* kv_lens,
                                            const void* token_seq, void* out, int N, int nq, int nkv, int d,
                                            int page_size, int64_t page_stride, int max_pages, int window,
-                                           float scale, int dtype, hipStream_t stream) {
+                                           float scale, int dtype, const void* sinks, hipStream_t stream) {
     if (N <= 0) return 0;
     if (d > ATT_MAX_R * LLE_WAVE) return (int)hipErrorInvalidValue;
     dim3 grid(N, nq);
@@ -176,12 +179,12 @@ extern "C" int lle_paged_attention_generic(const void* q, const void* kv_layer, 
         paged_attention_generic_kernel<float><<<grid, ATT_WAVES * LLE_WAVE, 0, stream>>>(
             (const float*)q, (const float*)kv_layer, (const int32_t*)block_tables, (const int32_t*)seq_slots,
             (const int32_t*)cu_tokens, (const int32_t*)kv_lens, (const int32_t*)token_seq, (float*)out, nq, nkv, d,
-            page_size, page_stride, max_pages, window, scale);
+            page_size, page_stride, max_pages, window, scale, (const float*)sinks);
     else
         paged_attention_generic_kernel<bf16_t><<<grid, ATT_WAVES * LLE_WAVE, 0, stream>>>(
             (const bf16_t*)q, (const bf16_t*)kv_layer, (const int32_t*)block_tables, (const int32_t*)seq_slots,
             (const int32_t*)cu_tokens, (const int32_t*)kv_lens, (const int32_t*)token_seq, (bf16_t*)out, nq, nkv,
-            d, page_size, page_stride, max_pages, window, scale);
+            d, page_size, page_stride, max_pages, window, scale, (const float*)sinks);
     LLE_RETURN_LAUNCH_STATUS();
 }
 
@@ -690,7 +693,7 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int ws_stride, int nq, int nkv, int P, int64_t page_stride, int max_pages,
-    int window, float scale_log2, FusedQKV fused) {
+    int window, float scale_log2, FusedQKV fused, const float* __restrict__ sinks) {
     constexpr int D = DK * 32;
     extern __shared__ float smem[];  // [waves][16][D] acc, then [waves][16] m, [waves][16] l
     float* s_o = smem;
@@ -793,6 +796,7 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
         const int t = r / G, g = r - t * G;
         const int64_t head_row = (int64_t)(q_start + t) * nq + kvh * G + g;
         if (nsplit == 1) {
+            if (sinks) den += exp2f(sinks[kvh * G + g] * 1.44269504088896340736f - big);  // (a sink: a place in the sum without a value)
             out[head_row * D + e] = (bf16_t)(num / den);
         } else {
             ws_o[(head_row * ws_stride + split) * D + e] = num;
@@ -813,7 +817,8 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
                                                                 const int32_t* __restrict__ cu_tokens,
                                                                 const int32_t* __restrict__ token_seq,
                                                                 bf16_t* __restrict__ out, int nq, int nkv, int D,
-                                                                int nsplit_decode, int nsplit_prefill) {
+                                                                int nsplit_decode, int nsplit_prefill,
+                                                                const float* __restrict__ sinks) {
     const int64_t tok = blockIdx.x;
     const int h = blockIdx.y;
     int nsplit = nsplit_decode;
@@ -835,7 +840,8 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
     const float m = lane < nsplit ? ml.x : NEG_BIG, l = lane < nsplit ? ml.y : 0.f;
     const float big = wave_max(m);
     const float f = exp2f(m - big);  // 0 for lanes without a split (l = 0 there anyway)
-    const float den = wave_sum(l * f);
+    float den = wave_sum(l * f);
+    if (sinks) den += exp2f(sinks[h] * 1.44269504088896340736f - big);  // (a sink: a place in the sum without a value)
     // every lane needs every split's factor, also those of lanes that have no element below
     __shared__ float s_f[LLE_WAVE];
     s_f[lane] = f;
@@ -898,7 +904,7 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int ws_stride, int nsplit, int nq, int nkv, int P, int64_t page_stride, int max_pages,
-    int window, float scale_log2, int complement_order) {
+    int window, float scale_log2, int complement_order, const float* __restrict__ sinks) {
     constexpr int D = DK * 32;
     static_assert(PRE_RT <= PRE_RT_OF(DK), "the accumulators of two row tiles fit the registers up to heads of 128");
     constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT;
@@ -1194,7 +1200,8 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
             continue;
         }
         bf16_t* dst = out + head_row * D;
-        const float inv = 1.0f / st.l[t];
+        // (a sink: a place in the sum without a value)
+        const float inv = 1.0f / (sinks ? st.l[t] + exp2f(sinks[kvh * G + g] * 1.44269504088896340736f - st.m[t]) : st.l[t]);
 #pragma unroll
         for (int n = 0; n < 2 * DK; ++n) {
             bf16x4 v;
@@ -1230,7 +1237,7 @@ __global__ __launch_bounds__(F32_WAVES* LLE_WAVE) void mfma_f32_attention_kernel
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, float* __restrict__ out, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int nsplit, int nq, int nkv, int P, int64_t page_stride, int max_pages, int window,
-    float scale_log2) {
+    float scale_log2, const float* __restrict__ sinks) {
     constexpr int D = 16 * DQ;
     extern __shared__ float smem[];  // [waves][16][D] acc, then [waves][16] m, [waves][16] l
     float* s_o = smem;
@@ -1367,7 +1374,8 @@ __global__ __launch_bounds__(F32_WAVES* LLE_WAVE) void mfma_f32_attention_kernel
             }
             return;
         }
-        const float inv = 1.0f / l;
+        // (a sink: a place in the sum without a value)
+        const float inv = 1.0f / (sinks ? l + exp2f(sinks[kvh * G + g] * 1.44269504088896340736f - m) : l);
 #pragma unroll
         for (int n = 0; n < DQ; ++n) *(f32x4*)(out + head_row * D + 16 * n + 4 * c) = o[n] * inv;
         return;
@@ -1397,6 +1405,7 @@ __global__ __launch_bounds__(F32_WAVES* LLE_WAVE) void mfma_f32_attention_kernel
         const int t = r / G, gg = r - t * G;
         const int64_t hr = (int64_t)(q_start + t) * nq + kvh * G + gg;
         if (nsplit == 1) {
+            if (sinks) den += exp2f(sinks[kvh * G + gg] * 1.44269504088896340736f - big);
             out[hr * D + e] = num / den;
         } else {
             ws_o[(hr * nsplit + split) * D + e] = num;
@@ -1411,7 +1420,8 @@ __global__ __launch_bounds__(F32_WAVES* LLE_WAVE) void mfma_f32_attention_kernel
 // merges the key splits of the kernel above: grid = (tokens, q heads), one wavefront each
 __global__ __launch_bounds__(LLE_WAVE) void f32_combine_kernel(const float* __restrict__ ws_o,
                                                                const float* __restrict__ ws_ml, int nsplit,
-                                                               float* __restrict__ out, int nq, int D) {
+                                                               float* __restrict__ out, int nq, int D,
+                                                               const float* __restrict__ sinks) {
     const int64_t head_row = (int64_t)blockIdx.x * nq + blockIdx.y;
     const int lane = threadIdx.x;
     __shared__ float s_f[LLE_WAVE];
@@ -1419,7 +1429,8 @@ __global__ __launch_bounds__(LLE_WAVE) void f32_combine_kernel(const float* __re
     const float m = lane < nsplit ? ml.x : NEG_BIG, l = lane < nsplit ? ml.y : 0.f;
     const float big = wave_max(m);
     const float f = exp2f(m - big);
-    const float den = wave_sum(l * f);
+    float den = wave_sum(l * f);
+    if (sinks) den += exp2f(sinks[blockIdx.y] * 1.44269504088896340736f - big);
     s_f[lane] = f;
     __syncthreads();
     const float* o = ws_o + head_row * nsplit * D;
@@ -1438,7 +1449,8 @@ extern "C" int lle_paged_attention_mfma_f32(const void* q, const void* kv_layer,
                                             const void* seq_slots, const void* cu_tokens, const void* kv_lens,
                                             void* out, void* ws_o, void* ws_ml, int N, int S, int nq, int nkv, int d,
                                             int page_size, int64_t page_stride, int max_pages, int window,
-                                            float scale, int row_blocks, int nsplit, hipStream_t stream) {
+                                            float scale, int row_blocks, int nsplit, const void* sinks,
+                                            hipStream_t stream) {
     if (N <= 0) return 0;
     if (d % 16 != 0 || d > 256 || d <= 0 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
     if (S > 65535 || nkv <= 0 || row_blocks < 1 || nsplit < 1 || nsplit > 64 || (int64_t)row_blocks * nsplit > 65535)
@@ -1457,7 +1469,7 @@ extern "C" int lle_paged_attention_mfma_f32(const void* q, const void* kv_layer,
         mfma_f32_attention_kernel<DQV><<<grid, F32_WAVES * LLE_WAVE, smem, stream>>>(                             \
             (const float*)q, (const float*)kv_layer, (const int32_t*)block_tables, (const int32_t*)seq_slots,     \
             (const int32_t*)cu_tokens, (const int32_t*)kv_lens, (float*)out, (float*)ws_o, (float*)ws_ml, nsplit, \
-            nq, nkv, page_size, page_stride, max_pages, window, scale_log2);                                      \
+            nq, nkv, page_size, page_stride, max_pages, window, scale_log2, (const float*)sinks);                \
         break;
     switch (d / 16) {
         LLE_F32_CASE(1) LLE_F32_CASE(2) LLE_F32_CASE(3) LLE_F32_CASE(4) LLE_F32_CASE(5) LLE_F32_CASE(6)
@@ -1467,7 +1479,7 @@ extern "C" int lle_paged_attention_mfma_f32(const void* q, const void* kv_layer,
 #undef LLE_F32_CASE
     if (nsplit > 1)
         f32_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>((const float*)ws_o, (const float*)ws_ml, nsplit,
-                                                                 (float*)out, nq, d);
+                                                                 (float*)out, nq, d, (const float*)sinks);
     return (int)hipGetLastError();
 }
 
@@ -1488,7 +1500,7 @@ template <int DK, bool FUSED>
 static int launch_decode(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_tables, const int32_t* seq_slots,
                          const int32_t* cu_tokens, const int32_t* kv_lens, bf16_t* out, float* ws_o, float* ws_ml,
                          int ws_stride, int S, int nq, int nkv, int P, int64_t page_stride, int max_pages, int window,
-                         float scale_log2, int nsplit, const FusedQKV& fused, hipStream_t stream) {
+                         float scale_log2, int nsplit, const FusedQKV& fused, const float* sinks, hipStream_t stream) {
     constexpr int D = DK * 32;
     const size_t smem = (size_t)(DEC_WAVES * 16 * D + 2 * DEC_WAVES * 16) * sizeof(float);
     if (smem > 64 * 1024) {
@@ -1498,7 +1510,7 @@ static int launch_decode(const bf16_t* q, bf16_t* kv_layer, const int32_t* block
     }
     mfma_decode_kernel<DK, FUSED><<<dim3(S, nkv, nsplit), DEC_WAVES * LLE_WAVE, smem, stream>>>(
         q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nq, nkv, P,
-        page_stride, max_pages, window, scale_log2, fused);
+        page_stride, max_pages, window, scale_log2, fused, sinks);
     return 0;
 }
 
@@ -1533,7 +1545,7 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
                        const int32_t* token_seq, bf16_t* out, float* ws_o, float* ws_ml, int N, int S, int nq,
                        int nkv, int P, int64_t page_stride, int max_pages, int window, float scale_log2,
                        int run_decode, int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
-                       int prefill_form, const FusedQKV& fused, hipStream_t stream) {
+                       int prefill_form, const FusedQKV& fused, const float* sinks, hipStream_t stream) {
     constexpr int D = DK * 32;
     const int G = nq / nkv;
     if (!run_decode) nsplit_decode = 1;
@@ -1553,14 +1565,14 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
         if constexpr (DK % 2 == 0) {
             e = fused.qkv ? launch_decode<DK, true>(q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o,
                                                     ws_ml, ws_stride, S, nq, nkv, P, page_stride, max_pages, window,
-                                                    scale_log2, nsplit_decode, fused, stream)
+                                                    scale_log2, nsplit_decode, fused, sinks, stream)
                           : launch_decode<DK, false>(q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out,
                                                      ws_o, ws_ml, ws_stride, S, nq, nkv, P, page_stride, max_pages,
-                                                     window, scale_log2, nsplit_decode, fused, stream);
+                                                     window, scale_log2, nsplit_decode, fused, sinks, stream);
         } else {
             e = launch_decode<DK, false>(q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml,
                                          ws_stride, S, nq, nkv, P, page_stride, max_pages, window, scale_log2,
-                                         nsplit_decode, fused, stream);
+                                         nsplit_decode, fused, sinks, stream);
         }
         if (e != 0) {
             if (lane) (void)hipStreamSynchronize(lane->stream);
@@ -1586,7 +1598,7 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
             const int64_t workgroups = (int64_t)nkv * blocks * nsplit_prefill * S;
             mfma_prefill_kernel<DK, RT, WAVES><<<dim3(nkv, blocks * nsplit_prefill, S), WAVES * LLE_WAVE, 0, stream>>>(
                 q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nsplit_prefill,
-                nq, nkv, P, page_stride, max_pages, window, scale_log2, workgroups <= 2 * compute_units() ? 1 : 0);
+                nq, nkv, P, page_stride, max_pages, window, scale_log2, workgroups <= 2 * compute_units() ? 1 : 0, sinks);
         };
         using Four = std::integral_constant<int, 4>;
         if (DK == 4 && prefill_form == 3) {
@@ -1605,7 +1617,7 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
     if (ws_stride > 1)  // a batch of one kind needs no look at the tokens' requests
         mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(
             ws_o, ws_ml, ws_stride, cu_tokens, token_seq, out, nq, nkv, D, run_decode ? nsplit_decode : nsplit_prefill,
-            run_prefill ? nsplit_prefill : nsplit_decode);
+            run_prefill ? nsplit_prefill : nsplit_decode, sinks);
     return (int)hipGetLastError();
 }
 
@@ -1619,7 +1631,7 @@ static int paged_attention_mfma(const void* q, void* kv_layer, const void* block
                                 void* ws_o, void* ws_ml, int N, int S, int nq, int nkv, int d, int page_size,
                                 int64_t page_stride, int max_pages, int window, float scale, int run_decode,
                                 int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
-                                int prefill_form, const FusedQKV& fused, hipStream_t stream) {
+                                int prefill_form, const FusedQKV& fused, const float* sinks, hipStream_t stream) {
     if (N <= 0) return 0;
     if (d % 32 != 0 || d > 256 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
     if (S > 65535 || nkv > 65535 || page_stride < 0 || page_stride >= ((int64_t)1 << 32)) return (int)hipErrorInvalidValue;
@@ -1632,7 +1644,7 @@ static int paged_attention_mfma(const void* q, void* kv_layer, const void* block
                                 (const int32_t*)seq_slots, (const int32_t*)cu_tokens, (const int32_t*)kv_lens,      \
                                 (const int32_t*)token_seq, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, N, S, nq, nkv, \
                                 page_size, page_stride, max_pages, window, scale_log2, run_decode, nsplit_decode,   \
-                                run_prefill, nsplit_prefill, max_q_len, prefill_form, fused, stream);
+                                run_prefill, nsplit_prefill, max_q_len, prefill_form, fused, sinks, stream);
     switch (d / 32) {
         LLE_ATT_CASE(1)
         LLE_ATT_CASE(2)
@@ -1652,12 +1664,13 @@ extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, con
                                         const void* token_seq, void* out, void* ws_o, void* ws_ml, int N, int S,
                                         int nq, int nkv, int d, int page_size, int64_t page_stride, int max_pages,
                                         int window, float scale, int run_decode, int nsplit_decode, int run_prefill,
-                                        int nsplit_prefill, int max_q_len, int prefill_form,
+                                        int nsplit_prefill, int max_q_len, int prefill_form, const void* sinks,
                                         hipStream_t stream) {
     const FusedQKV none = {};
     return paged_attention_mfma(q, (void*)kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, token_seq, out, ws_o,
                                 ws_ml, N, S, nq, nkv, d, page_size, page_stride, max_pages, window, scale, run_decode,
-                                nsplit_decode, run_prefill, nsplit_prefill, max_q_len, prefill_form, none, stream);
+                                nsplit_decode, run_prefill, nsplit_prefill, max_q_len, prefill_form, none,
+                                (const float*)sinks, stream);
 }
 
 // Decode steps only (every request has at most 16 / group tokens), head_dim a multiple of 64, a
@@ -1686,5 +1699,5 @@ extern "C" int lle_qk_norm_rope_attention_decode(const void* qkv, const void* sl
     fused.write_kv = write_kv;
     return paged_attention_mfma(nullptr, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, token_seq, out, ws_o,
                                 ws_ml, N, S, nq, nkv, d, page_size, page_stride, max_pages, window, scale, 1,
-                                nsplit_decode, 0, 1, 1, 0, fused, stream);
+                                nsplit_decode, 0, 1, 1, 0, fused, nullptr, stream);
 }

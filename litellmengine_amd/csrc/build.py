@@ -35,6 +35,7 @@ LIBRARIES: Dict[str, List[str]] = {
     "recurrent": ["recurrent.hip"],
     "latent": ["latent.hip"],
     "moe": ["moe.hip"],
+    "wkv": ["wkv.hip"],
     "probe": ["probe.hip"],
 }
 # libraries without GPU code: compiled with the host's C++ compiler

@@ -170,3 +170,52 @@ extern "C" int lle_scale(void* x, int64_t total, float factor, hipStream_t strea
     scale_kernel<<<(int)blocks, 256, 0, stream>>>((float*)x, total, factor);
     LLE_RETURN_LAUNCH_STATUS();
 }
+
+// out[n, h, :vdim] = a[n, h, :vdim] * sigmoid(gates[n, col0 + h]): a gate per head on an attention's result
+// (`a` rows hold heads of D >= vdim elements; what lies past vdim is dropped)
+template <typename T>
+__global__ __launch_bounds__(256) void head_gate_kernel(const T* __restrict__ a, const T* __restrict__ gates, int gate_cols,
+                                                         int col0, T* __restrict__ out, int64_t total, int heads, int D,
+                                                         int vdim) {
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int e = (int)(idx % vdim);
+        const int64_t nh = idx / vdim;
+        const int h = (int)(nh % heads);
+        const int64_t n = nh / heads;
+        const float g = to_f32<T>(gates[n * gate_cols + col0 + h]);
+        out[idx] = from_f32<T>(to_f32<T>(a[nh * D + e]) / (1.0f + expf(-g)));
+    }
+}
+
+extern "C" int lle_head_gate(const void* a, const void* gates, int gate_cols, int col0, void* out, int N, int heads, int D,
+                             int vdim, int dtype, hipStream_t stream) {
+    const int64_t total = (int64_t)N * heads * vdim;
+    if (total <= 0) return 0;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == LLE_F32)
+        head_gate_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)a, (const float*)gates, gate_cols, col0,
+                                                                  (float*)out, total, heads, D, vdim);
+    else
+        head_gate_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)gates, gate_cols, col0,
+                                                                   (bf16_t*)out, total, heads, D, vdim);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// x = tanh(x) in place
+template <typename T>
+__global__ __launch_bounds__(256) void tanh_kernel(T* __restrict__ x, int64_t total) {
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x)
+        x[idx] = from_f32<T>(tanhf(to_f32<T>(x[idx])));
+}
+
+extern "C" int lle_tanh(void* x, int64_t total, int dtype, hipStream_t stream) {
+    if (total <= 0) return 0;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == LLE_F32) tanh_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)x, total);
+    else tanh_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)x, total);
+    LLE_RETURN_LAUNCH_STATUS();
+}

@@ -4,6 +4,8 @@
 //   ids, gains = top-k of (logits + bias), gains = softmax over the chosen logits     moe_route
 //   act[p]   = silu(Wg[e_p] x_n) * (Wu[e_p] x_n)      p = (token n, k-th choice)      moe_gate_up
 //   out[n]   = sum_k gains[n, k] * Wd[e_(n,k)] act[(n, k)]        32-bit              moe_down
+// An id from E on (E: the experts that have weights) names an identity expert: its result is its input,
+// so such a pair adds gains[n, k] * x_n and takes no part in the products.
 //
 // Few tokens (decoding), or float32: every (token, choice) pair streams the rows of its expert's
 // weights, a wavefront per output element.  Many bfloat16 tokens (prompt portions, large batches): the
@@ -75,6 +77,101 @@ extern "C" int lle_moe_route(const void* logits, const void* bias, void* ids, vo
     LLE_RETURN_LAUNCH_STATUS();
 }
 
+
+// A router whose scores are the softmax over ALL experts and whose choice is limited to groups: one wavefront per
+// token.  scores s = softmax(logits); choice scores c = s + correction; the experts form `groups` equal groups of
+// neighbours, a group's score is its largest c, and only the `keep` best groups' experts can be chosen (the lower
+// index wins a tie, among groups and among experts); gains = s of the chosen / (their sum + 1e-20).
+// Dynamic LDS: per wavefront E scores, E choice scores and `groups` group scores.
+__global__ __launch_bounds__(256) void moe_route_grouped_kernel(const float* __restrict__ logits,
+                                                                 const float* __restrict__ correction,
+                                                                 int32_t* __restrict__ ids, float* __restrict__ gains,
+                                                                 int N, int E, int top, int groups, int keep) {
+    extern __shared__ float route_smem[];
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    const int n = min(blockIdx.x * (blockDim.x / LLE_WAVE) + wave, N - 1);  // (a wavefront past the end repeats the last token)
+    float* s = route_smem + (int64_t)wave * (2 * E + groups);
+    float* c = s + E;
+    float* best = c + E;
+    const float* row = logits + (int64_t)n * E;
+    float big = -INFINITY;
+    for (int e = lane; e < E; e += LLE_WAVE) big = fmaxf(big, row[e]);
+    big = wave_max(big);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += LLE_WAVE) {
+        const float x = expf(row[e] - big);
+        s[e] = x;
+        sum += x;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += LLE_WAVE) {
+        const float x = s[e] / sum;
+        s[e] = x;
+        c[e] = x + correction[e];
+    }
+    __syncthreads();
+    const int size = E / groups;
+    for (int g = lane; g < groups; g += LLE_WAVE) {
+        float b = c[g * size];
+        for (int i = 1; i < size; ++i) b = fmaxf(b, c[g * size + i]);
+        best[g] = b;
+    }
+    __syncthreads();
+    if (keep < groups) {
+        for (int g = lane; g < groups; g += LLE_WAVE) {
+            int ahead = 0;  // groups that come before this one
+            for (int o = 0; o < groups; ++o) ahead += (best[o] > best[g] || (best[o] == best[g] && o < g)) ? 1 : 0;
+            if (ahead >= keep)
+                for (int i = 0; i < size; ++i) c[g * size + i] = -INFINITY;
+        }
+        __syncthreads();
+    }
+    int chosen[MOE_MAX_TOP];  // the same in every lane
+    float total = 0.f;
+    for (int k = 0; k < top; ++k) {
+        int pick = 0x7fffffff;
+        float bv = -INFINITY;
+        for (int e = lane; e < E; e += LLE_WAVE) {
+            bool taken = false;
+            for (int j = 0; j < k; ++j) taken |= chosen[j] == e;
+            const float v = c[e];
+            if (!taken && (pick == 0x7fffffff || v > bv)) {  // (e rises: an equal value later loses)
+                pick = e;
+                bv = v;
+            }
+        }
+#pragma unroll
+        for (int o = LLE_WAVE / 2; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, LLE_WAVE);
+            const int oe = __shfl_xor(pick, o, LLE_WAVE);
+            if (oe != 0x7fffffff && (pick == 0x7fffffff || ov > bv || (ov == bv && oe < pick))) {
+                bv = ov;
+                pick = oe;
+            }
+        }
+        chosen[k] = pick;
+        total += s[pick];
+    }
+    if (lane != 0) return;
+    for (int k = 0; k < top; ++k) {
+        ids[(int64_t)n * top + k] = chosen[k];
+        gains[(int64_t)n * top + k] = s[chosen[k]] / (total + 1e-20f);
+    }
+}
+
+extern "C" int lle_moe_route_grouped(const void* logits, const void* correction, void* ids, void* gains, int N, int E,
+                                     int top, int groups, int keep, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (top <= 0 || top > MOE_MAX_TOP || top > E || groups <= 0 || E % groups || keep <= 0 || keep > groups ||
+        top > keep * (E / groups))
+        return (int)hipErrorInvalidValue;
+    const size_t lds = (size_t)4 * (2 * E + groups) * sizeof(float);
+    if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
+    moe_route_grouped_kernel<<<(N + 3) / 4, 256, lds, stream>>>((const float*)logits, (const float*)correction,
+                                                                   (int32_t*)ids, (float*)gains, N, E, top, groups, keep);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
 typedef bf16_t wbf16x8 __attribute__((ext_vector_type(8)));
 
 // sum over K of a[k] b[k] by one wavefront, every lane gets it; 16-byte loads where the rows allow them
@@ -103,11 +200,12 @@ __device__ __forceinline__ float wave_dot(const T* __restrict__ a, const T* __re
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ x, const int32_t* __restrict__ ids,
                                                            const T* __restrict__ gate_up, T* __restrict__ act, int top,
-                                                           int F, int K) {
+                                                           int F, int K, int E) {
     const int p = blockIdx.x;
     const int f = blockIdx.y * 4 + threadIdx.x / LLE_WAVE;
     if (f >= F) return;
     const int e = ids[p];
+    if (e >= E) return;  // an identity expert: nothing to multiply
     const T* xr = x + (int64_t)(p / top) * K;
     const T* w = gate_up + (int64_t)e * 2 * F * K;
     const float g = wave_dot<T>(xr, w + (int64_t)f * K, K);
@@ -119,37 +217,44 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
 template <typename T>
 __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act, const int32_t* __restrict__ ids,
                                                         const float* __restrict__ gains, const T* __restrict__ down,
-                                                        float* __restrict__ out, int top, int F, int H) {
+                                                        const T* __restrict__ x, float* __restrict__ out, int top, int F,
+                                                        int H, int E) {
     const int n = blockIdx.x;
     const int o = blockIdx.y * 4 + threadIdx.x / LLE_WAVE;
     if (o >= H) return;
     float total = 0.f;
     for (int k = 0; k < top; ++k) {
         const int p = n * top + k;
-        const T* w = down + ((int64_t)ids[p] * H + o) * F;
+        const int e = ids[p];
+        if (e >= E) {  // (the same for the whole wavefront)
+            total += gains[p] * to_f32<T>(x[(int64_t)n * H + o]);
+            continue;
+        }
+        const T* w = down + ((int64_t)e * H + o) * F;
         total += gains[p] * wave_dot<T>(act + (int64_t)p * F, w, F);
     }
     if (threadIdx.x % LLE_WAVE == 0) out[(int64_t)n * H + o] = total;
 }
 
-// x [N, K], ids/gains [N, top], gate_up [E, 2 F, K], down [E, H, F], act [N top, F] (scratch), out float32 [N, H]
+// x [N, K], ids/gains [N, top], gate_up [E, 2 F, K], down [E, H, F], act [N top, F] (scratch), out float32 [N, H];
+// ids from E on are identity experts (then H = K)
 extern "C" int lle_moe_experts(const void* x, const void* ids, const void* gains, const void* gate_up,
-                               const void* down, void* act, void* out, int N, int top, int F, int K, int H, int dtype,
-                               hipStream_t stream) {
+                               const void* down, void* act, void* out, int N, int top, int E, int F, int K, int H,
+                               int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
     if (top <= 0 || (int64_t)N * top > 0x7fffffff) return (int)hipErrorInvalidValue;
     const dim3 g1(N * top, (F + 3) / 4), g2(N, (H + 3) / 4);
     if (g1.y > 65535 || g2.y > 65535) return (int)hipErrorInvalidValue;
     if (dtype == LLE_F32) {
         moe_gate_up_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const int32_t*)ids, (const float*)gate_up,
-                                                           (float*)act, top, F, K);
+                                                           (float*)act, top, F, K, E);
         moe_down_kernel<float><<<g2, 256, 0, stream>>>((const float*)act, (const int32_t*)ids, (const float*)gains,
-                                                        (const float*)down, (float*)out, top, F, H);
+                                                        (const float*)down, (const float*)x, (float*)out, top, F, H, E);
     } else {
         moe_gate_up_kernel<bf16_t><<<g1, 256, 0, stream>>>((const bf16_t*)x, (const int32_t*)ids,
-                                                            (const bf16_t*)gate_up, (bf16_t*)act, top, F, K);
+                                                            (const bf16_t*)gate_up, (bf16_t*)act, top, F, K, E);
         moe_down_kernel<bf16_t><<<g2, 256, 0, stream>>>((const bf16_t*)act, (const int32_t*)ids, (const float*)gains,
-                                                         (const bf16_t*)down, (float*)out, top, F, H);
+                                                         (const bf16_t*)down, (const bf16_t*)x, (float*)out, top, F, H, E);
     }
     LLE_RETURN_LAUNCH_STATUS();
 }
@@ -187,7 +292,7 @@ __global__ __launch_bounds__(256) void moe_count_kernel(const int32_t* __restric
     local[threadIdx.x] = 0;
     __syncthreads();
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
-    if (p < pairs) atomicAdd(&local[ids[p]], 1);
+    if (p < pairs && ids[p] < E) atomicAdd(&local[ids[p]], 1);  // (identity experts have no rows)
     __syncthreads();
     if (threadIdx.x < E && local[threadIdx.x]) atomicAdd(&counts[threadIdx.x], local[threadIdx.x]);
 }
@@ -221,13 +326,17 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* __restric
     int e = 0, mine = 0;
     if (p < pairs) {
         e = ids[p];
-        mine = atomicAdd(&local[e], 1);
+        if (e < E) mine = atomicAdd(&local[e], 1);
     }
     __syncthreads();
     if (threadIdx.x < E && local[threadIdx.x])
         local[threadIdx.x] = plan[2 * E + threadIdx.x] + atomicAdd(&plan[E + threadIdx.x], local[threadIdx.x]);
     __syncthreads();
     if (p >= pairs) return;
+    if (e >= E) {  // an identity expert: the pair has no row
+        place[p] = -1;
+        return;
+    }
     const int row = local[e] + mine;
     order[row] = p;
     place[p] = row;
@@ -404,16 +513,22 @@ __global__ __launch_bounds__(256, 2) void moe_down_tile_kernel(const bf16_t* __r
     }
 }
 
-// out[n, :] = sum_k gains[n, k] * y[place[n top + k], :], in the order of k
+// out[n, :] = sum_k gains[n, k] * y[place[n top + k], :], in the order of k; a pair without a row (an identity
+// expert's) adds its token's own x row
 __global__ __launch_bounds__(256) void moe_gather_kernel(const float* __restrict__ y, const int32_t* __restrict__ place,
-                                                          const float* __restrict__ gains, float* __restrict__ out,
-                                                          int top, int H) {
+                                                          const float* __restrict__ gains, const bf16_t* __restrict__ x,
+                                                          float* __restrict__ out, int top, int H) {
     const int n = blockIdx.x;
     for (int o = threadIdx.x * 4; o < H; o += blockDim.x * 4) {
         mf32x4 total = mf32x4{0.f, 0.f, 0.f, 0.f};
         for (int k = 0; k < top; ++k) {
             const int p = n * top + k;
-            total += gains[p] * *(const mf32x4*)(y + (int64_t)place[p] * H + o);
+            if (place[p] < 0) {
+                const mbf16x4 xv = *(const mbf16x4*)(x + (int64_t)n * H + o);
+                total += gains[p] * mf32x4{(float)xv[0], (float)xv[1], (float)xv[2], (float)xv[3]};
+            } else {
+                total += gains[p] * *(const mf32x4*)(y + (int64_t)place[p] * H + o);
+            }
         }
         *(mf32x4*)(out + (int64_t)n * H + o) = total;
     }
@@ -442,7 +557,7 @@ extern "C" int lle_moe_experts_tiled(const void* x, const void* ids, const void*
         tiles, fb);
     moe_down_tile_kernel<<<8 * ((tiles * hb + 7) / 8), 256, 0, stream>>>(
         (const bf16_t*)act, (const int32_t*)plan, (const bf16_t*)down, (float*)y, E, F, H, tiles, hb);
-    moe_gather_kernel<<<N, 256, 0, stream>>>((const float*)y, (const int32_t*)place, (const float*)gains, (float*)out,
-                                                top, H);
+    moe_gather_kernel<<<N, 256, 0, stream>>>((const float*)y, (const int32_t*)place, (const float*)gains,
+                                                (const bf16_t*)x, (float*)out, top, H);
     LLE_RETURN_LAUNCH_STATUS();
 }

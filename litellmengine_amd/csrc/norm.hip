@@ -371,3 +371,83 @@ extern "C" int lle_rmsnorm_add(void* hidden, const void* y, int y_dtype, const v
                                                                weight_dtype, (bf16_t*)out, H, eps);
     LLE_RETURN_LAUNCH_STATUS();
 }
+
+// For arrangements whose sublayers run side by side on one norm's result and whose sum enters the stream
+// times a constant: hidden[r] += mult * (a[r] (+ b[r])) in 32-bit and in place, then out[r] = norm(hidden[r]) * w.
+// `a`, `b` hold float32 or bfloat16, each said by its own code.  With `rows` only those rows are read, row
+// rows[r] gives out[r], and `hidden` is left alone.  The new row waits in registers between the sum of
+// squares and the scaling (rows up to 256 x 4 x SA_CHUNKS wide and a multiple of 4; a plain loop otherwise).
+#define SA_CHUNKS 8
+template <typename TO>
+__global__ __launch_bounds__(256) void scaled_add_rmsnorm_kernel(float* __restrict__ hidden, const void* __restrict__ a,
+                                                                  int a_dtype, const void* __restrict__ b, int b_dtype,
+                                                                  float mult, const int32_t* __restrict__ rows,
+                                                                  const void* __restrict__ weight, int weight_dtype,
+                                                                  TO* __restrict__ out, int H, float eps) {
+    __shared__ float red[16];
+    const int64_t r = rows ? rows[blockIdx.x] : blockIdx.x;
+    const int64_t at = r * H, to = (int64_t)blockIdx.x * H;
+    float ss = 0.f;
+    if (H % 4 == 0 && H <= 256 * 4 * SA_CHUNKS) {
+        float4 keep[SA_CHUNKS];
+#pragma unroll
+        for (int c = 0; c < SA_CHUNKS; ++c) {
+            const int i = (c * 256 + threadIdx.x) * 4;
+            if (i < H) {
+                float4 h = *(const float4*)(hidden + at + i);
+                float v[4] = {h.x, h.y, h.z, h.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float d = load_as_f32(a, at + i + e, a_dtype);
+                    if (b) d += load_as_f32(b, at + i + e, b_dtype);
+                    v[e] += mult * d;
+                    ss += v[e] * v[e];
+                }
+                keep[c] = make_float4(v[0], v[1], v[2], v[3]);
+                if (!rows) *(float4*)(hidden + at + i) = keep[c];
+            }
+        }
+        ss = block_sum(ss, red);
+        const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+        for (int c = 0; c < SA_CHUNKS; ++c) {
+            const int i = (c * 256 + threadIdx.x) * 4;
+            if (i < H) {
+                const float v[4] = {keep[c].x, keep[c].y, keep[c].z, keep[c].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out[to + i + e] = from_f32<TO>(v[e] * inv * load_as_f32(weight, i + e, weight_dtype));
+            }
+        }
+        return;
+    }
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float d = load_as_f32(a, at + i, a_dtype);
+        if (b) d += load_as_f32(b, at + i, b_dtype);
+        const float v = hidden[at + i] + mult * d;
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float d = load_as_f32(a, at + i, a_dtype);
+        if (b) d += load_as_f32(b, at + i, b_dtype);
+        const float v = hidden[at + i] + mult * d;
+        if (!rows) hidden[at + i] = v;
+        out[to + i] = from_f32<TO>(v * inv * load_as_f32(weight, i, weight_dtype));
+    }
+}
+
+// R = number of rows of `out` (all rows of `hidden`, or the length of `rows`)
+extern "C" int lle_scaled_add_rmsnorm(void* hidden, const void* a, int a_dtype, const void* b, int b_dtype, float mult,
+                                      const void* rows, const void* weight, int weight_dtype, void* out, int R, int H,
+                                      float eps, int out_dtype, hipStream_t stream) {
+    if (R <= 0) return 0;
+    if (out_dtype == LLE_F32)
+        scaled_add_rmsnorm_kernel<float><<<R, 256, 0, stream>>>((float*)hidden, a, a_dtype, b, b_dtype, mult,
+                                                                 (const int32_t*)rows, weight, weight_dtype, (float*)out, H, eps);
+    else
+        scaled_add_rmsnorm_kernel<bf16_t><<<R, 256, 0, stream>>>((float*)hidden, a, a_dtype, b, b_dtype, mult,
+                                                                  (const int32_t*)rows, weight, weight_dtype, (bf16_t*)out, H,
+                                                                  eps);
+    LLE_RETURN_LAUNCH_STATUS();
+}

@@ -424,8 +424,10 @@ class HipOps:
 
     def paged_attention(self, q, kv_layer, block_table, seq_slots, cu_tokens, kv_lens, token_seq,
                         window: Optional[int], scale: float, min_q_len: int = 0, max_q_len: int = 0,
-                        max_kv_len: int = 0) -> torch.Tensor:
-        """q [N, nq, d] against the pages -> [N, nq * d].  `min_q_len`, `max_q_len`
+                        max_kv_len: int = 0, sinks=None) -> torch.Tensor:
+        """q [N, nq, d] against the pages -> [N, nq * d].  `sinks` (float32 [nq], or None): every head's
+        softmax has one more place, with that score and no value: p_j = exp(s_j) / (exp(sink) + sum exp(s_j)).
+        `min_q_len`, `max_q_len`
         and `max_kv_len` are host-side bounds of this batch; they choose the kernels
         and the number of key splits, never the result.  bfloat16 with head_dim a
         multiple of 32 and a page size a multiple of 16 runs on the matrix cores;
@@ -444,6 +446,9 @@ class HipOps:
         S = seq_slots.shape[0]
         _need(cu_tokens.shape == (S + 1,) and kv_lens.shape == (S,), "cu_tokens [S + 1], kv_lens [S]")
         _need(block_table.dim() == 2, "block_table must be [slots, pages]")
+        if sinks is not None:
+            _dev(sinks, "sinks", torch.float32)
+            _need(sinks.shape == (nq,), "sinks must be [nq]")
         out = torch.empty((N, nq * d), dtype=q.dtype, device=q.device)
         win = int(window) if window else 0
         mfma = (q.dtype == torch.bfloat16 and d % 32 == 0 and page_size % 16 == 0 and max_q_len > 0
@@ -460,17 +465,17 @@ class HipOps:
                 ws_o = torch.empty((N * nq * ns * d,), dtype=torch.float32, device=q.device)
                 ws_ml = torch.empty((N * nq * ns * 2,), dtype=torch.float32, device=q.device)
             self._run("attention", "lle_paged_attention_mfma_f32",
-                      [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _I, _P],
+                      [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _I, _P, _P],
                       _ptr(q), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens), _ptr(kv_lens),
                       _ptr(out), _ptr(ws_o), _ptr(ws_ml), N, S, nq, nkv, d, page_size, kv_layer.stride(0),
-                      block_table.shape[1], win, float(scale), row_blocks, ns)
+                      block_table.shape[1], win, float(scale), row_blocks, ns, _ptr(sinks))
             return out
         if not mfma:
             self._run("attention", "lle_paged_attention_generic",
-                      [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _P],
+                      [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _P, _P],
                       _ptr(q), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens), _ptr(kv_lens),
                       _ptr(token_seq), _ptr(out), N, nq, nkv, d, page_size, kv_layer.stride(0), block_table.shape[1],
-                      win, float(scale), dtype_code(q.dtype))
+                      win, float(scale), dtype_code(q.dtype), _ptr(sinks))
             return out
         min_q_len = min_q_len or 1
         run_decode = min_q_len * group <= 16
@@ -486,11 +491,11 @@ class HipOps:
             ws_ml = torch.empty((N * nq * ns * 2,), dtype=torch.float32, device=q.device)
         self._run("attention", "lle_paged_attention_mfma",
                   [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _I, _I, _I, _I, _I,
-                   _P],
+                   _P, _P],
                   _ptr(q), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens), _ptr(kv_lens),
                   _ptr(token_seq), _ptr(out), _ptr(ws_o), _ptr(ws_ml), N, S, nq, nkv, d, page_size,
                   kv_layer.stride(0), block_table.shape[1], win, float(scale), int(run_decode), ns_decode,
-                  int(run_prefill), ns_prefill, max_q_len, row_tiles)
+                  int(run_prefill), ns_prefill, max_q_len, row_tiles, _ptr(sinks))
         return out
 
     def can_fuse_rope_attention(self, dtype, head_dim: int, rotary_dim: int, page_size: int, group: int,
@@ -901,11 +906,30 @@ class HipOps:
                   _ptr(gains), N, E, top)
         return ids, gains
 
+    def moe_route_grouped(self, logits, correction, top: int, groups: int = 1, keep: int = 1):
+        """float32 logits [N, E] -> (int32 ids [N, top], float32 gains [N, top]).  Scores are the softmax over
+        all E; the choice is made on score + correction [E], among the experts of the `keep` of `groups` equal
+        groups of neighbours whose largest choice score is largest (the lower index wins a tie); gains are the
+        chosen scores, without the correction, divided by their sum (+ 1e-20)."""
+        _dev(logits, "router logits", torch.float32)
+        _dev(correction, "router correction", torch.float32)
+        N, E = logits.shape
+        _need(correction.shape == (E,) and 0 < top <= min(E, 32), "a router picks between 1 and 32 of its experts")
+        _need(groups > 0 and E % groups == 0 and 0 < keep <= groups and top <= keep * (E // groups),
+              "the experts form equal groups, and the kept groups hold at least `top` experts")
+        _need(2 * E + groups <= 4096, "the router's kernel keeps its scores in LDS: at most about 2000 experts")
+        ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
+        gains = torch.empty((N, top), dtype=torch.float32, device=logits.device)
+        self._run("moe", "lle_moe_route_grouped", [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _ptr(logits),
+                  _ptr(correction), _ptr(ids), _ptr(gains), N, E, top, int(groups), int(keep))
+        return ids, gains
+
     MOE_TILED_MIN_PAIRS = 129  # (token, choice) pairs from which the sorted, tiled kernels take a bfloat16 step
 
     def moe_experts(self, x, ids, gains, gate_up, down) -> torch.Tensor:
         """x [N, K]; ids, gains [N, top]; gate_up [E, 2 F, K] (gate rows, then up rows); down [E, H, F] ->
-        float32 [N, H]: sum_k gains[n, k] * down[e] (silu(gate[e] x) * (up[e] x)), e = ids[n, k].
+        float32 [N, H]: sum_k gains[n, k] * down[e] (silu(gate[e] x) * (up[e] x)), e = ids[n, k].  An id from E on
+        names an identity expert, whose result is x itself (then H = K).
         Few pairs, or float32: every pair streams its expert's rows.  Many bfloat16 pairs: sorted by expert
         on the device, then tiles of 128 pairs of one expert on the matrix cores."""
         _dev(x, "x")
@@ -931,9 +955,154 @@ class HipOps:
                       _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(plan), order[0].data_ptr(),
                       order[1].data_ptr(), _ptr(act), _ptr(y), _ptr(out), N, top, E, F, K, H)
             return out
-        self._run("moe", "lle_moe_experts", [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
-                  _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(act), _ptr(out), N, top, F2 // 2,
+        self._run("moe", "lle_moe_experts", [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+                  _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(act), _ptr(out), N, top, E, F2 // 2,
                   K, H, dtype_code(x.dtype))
+        return out
+
+    # -- projections normed as a whole, sinks' attention gates -------------------------------
+    def proj_norm_rope_write(self, qkv, bias, slots, q_weight, k_weight, cos_sin, rotary_dim: int, eps: float, kv_layer,
+                             num_q_heads: int, num_kv_heads: int, dim: int, vdim: int, has_kv: bool = True,
+                             write_kv: bool = True) -> torch.Tensor:
+        """A row of qkv holds q [nq dim], then (`has_kv`) k [nkv dim] and v [nkv vdim], then columns that are
+        left alone; `bias` (or None) covers the whole row.  q and k are divided by the root mean square of their
+        whole projection, times q_weight [nq dim] / k_weight [nkv dim], then the first `rotary_dim` elements of
+        every head are rotated (half-split) by cos_sin [N, rotary_dim / 2, 2].  Returns q [N, nq, D] with
+        D = kv_layer.shape[4] >= max(dim, vdim), zeros past dim; K and V^T go to the pages `kv_layer`
+        [pages, 2, nkv, page_size, D] at `slots` [N] with zeros past dim and vdim."""
+        _dev(qkv, "qkv")
+        _dev(slots, "slots", torch.int32)
+        _dev(kv_layer, "kv_layer", qkv.dtype)
+        nq, nkv = num_q_heads, num_kv_heads
+        N, cols = qkv.shape
+        need = nq * dim + (nkv * (dim + vdim) if has_kv else 0)
+        _need(cols >= need, "qkv has too few columns")
+        _need(slots.shape == (N,), "slots must be [N]")
+        _need(kv_layer.dim() == 5 and kv_layer.shape[1] == 2 and kv_layer.shape[2] == nkv, "kv_layer must be [pages, 2, nkv, page_size, D]")
+        D, page_size = kv_layer.shape[4], kv_layer.shape[3]
+        _need(D >= max(dim, vdim), "the cache's heads are smaller than the model's")
+        _need(0 <= rotary_dim <= dim and rotary_dim % 2 == 0, "rotary_dim must be even and <= dim")
+        if bias is not None:
+            _dev(bias, "bias", qkv.dtype)
+            _need(bias.shape == (cols,), "bias must cover the whole row")
+        _dev(q_weight, "q norm weight")
+        _need(q_weight.shape == (nq * dim,), f"q norm weight must be [{nq * dim}]")
+        if has_kv:
+            _dev(k_weight, "k norm weight", q_weight.dtype)
+            _need(k_weight.shape == (nkv * dim,), f"k norm weight must be [{nkv * dim}]")
+        if rotary_dim > 0:
+            _dev(cos_sin, "cos_sin", torch.float32)
+            _need(cos_sin.shape == (N, rotary_dim // 2, 2), "cos_sin must be [N, rotary_dim / 2, 2]")
+        q_out = torch.empty((N, nq, D), dtype=qkv.dtype, device=qkv.device)
+        self._run("rope_kv", "lle_proj_norm_rope_write",
+                  [_P, _I, _P, _P, _P, _P, _I, _P, _I, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _I, _I, _I, _P],
+                  _ptr(qkv), cols, _ptr(bias), _ptr(slots), _ptr(q_weight), _ptr(k_weight) if has_kv else None,
+                  dtype_code(q_weight.dtype), _ptr(cos_sin) if rotary_dim > 0 else None, rotary_dim, float(eps),
+                  _ptr(q_out), _ptr(kv_layer), N, nq, nkv, dim, vdim, D, page_size, kv_layer.stride(0),
+                  1 if has_kv else 0, 1 if write_kv else 0, dtype_code(qkv.dtype))
+        return q_out
+
+    def head_gate(self, a, gates, col0: int, heads: int, vdim: int) -> torch.Tensor:
+        """a [N, heads * D], D >= vdim -> [N, heads * vdim]: head h's first vdim elements times
+        sigmoid(gates[n, col0 + h])."""
+        _dev(a, "a")
+        _dev(gates, "gates", a.dtype)
+        N = a.shape[0]
+        _need(a.dim() == 2 and a.shape[1] % heads == 0 and a.shape[1] // heads >= vdim, "a must be [N, heads * D], D >= vdim")
+        _need(gates.dim() == 2 and gates.shape[0] == N and 0 <= col0 and col0 + heads <= gates.shape[1], "gates [N, >= col0 + heads]")
+        out = torch.empty((N, heads * vdim), dtype=a.dtype, device=a.device)
+        self._run("elementwise", "lle_head_gate", [_P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _P], _ptr(a), _ptr(gates),
+                  gates.shape[1], int(col0), _ptr(out), N, heads, a.shape[1] // heads, vdim, dtype_code(a.dtype))
+        return out
+
+    def tanh_(self, x) -> torch.Tensor:
+        """x = tanh(x), in place."""
+        _dev(x, "x")
+        self._run("elementwise", "lle_tanh", [_P, _L, _I, _P], _ptr(x), x.numel(), dtype_code(x.dtype))
+        return x
+
+    def scaled_add_rmsnorm(self, hidden, a, b, mult: float, weight, eps: float, out_dtype, rows=None) -> torch.Tensor:
+        """hidden float32 [N, H] += mult * (a + b) in 32-bit and in place (`b` may be None; a, b [N, H],
+        float32 or bfloat16 each), then RMSNorm(hidden) * weight in `out_dtype`.  With `rows` (int32 [R]) only
+        those rows are read, row rows[r] gives row r of the result, and `hidden` is left alone."""
+        _dev(hidden, "hidden", torch.float32)
+        _dev(weight, "norm weight")
+        N, H = hidden.shape
+        _need(weight.shape == (H,), f"norm weight must be [{H}]")
+        for t, name in ((a, "a"), (b, "b")):
+            if t is not None:
+                _dev(t, name)
+                _need(t.shape == hidden.shape, f"{name} must have the shape of hidden")
+        R = N
+        if rows is not None:
+            _dev(rows, "rows", torch.int32)
+            R = rows.shape[0]
+        out = torch.empty((R, H), dtype=out_dtype, device=hidden.device)
+        self._run("norm", "lle_scaled_add_rmsnorm", [_P, _P, _I, _P, _I, _F, _P, _P, _I, _P, _I, _I, _F, _I, _P],
+                  _ptr(hidden), _ptr(a), dtype_code(a.dtype), _ptr(b), dtype_code(b.dtype) if b is not None else 0,
+                  float(mult), _ptr(rows), _ptr(weight), dtype_code(weight.dtype), _ptr(out), R, H, float(eps),
+                  dtype_code(out_dtype))
+        return out
+
+    # -- recurrence with a matrix state ------------------------------------------------------
+    def shift_mix(self, x, state, prev_offset: int, mu, token_seq, cu_tokens, seq_slots) -> torch.Tensor:
+        """x [N, W] -> [M, N, W]: out[m, n] = x[n] + (prev - x[n]) * mu[m], prev = x[n - 1], or for the first
+        token of a request's portion state[slot, prev_offset : prev_offset + W] (float32; what the step before
+        left there).  mu float32 [M, W]."""
+        _dev(x, "x")
+        _dev(state, "state", torch.float32)
+        _dev(mu, "mu", torch.float32)
+        for t, name in ((token_seq, "token_seq"), (cu_tokens, "cu_tokens"), (seq_slots, "seq_slots")):
+            _dev(t, name, torch.int32)
+        N, W = x.shape
+        M = mu.shape[0]
+        _need(mu.shape == (M, W) and state.dim() == 2 and prev_offset + W <= state.shape[1], "mu [M, W]; the state row holds W saved elements")
+        out = torch.empty((M, N, W), dtype=x.dtype, device=x.device)
+        self._run("wkv", "lle_shift_mix", [_P, _P, _L, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P], _ptr(x), _ptr(state),
+                  state.stride(0), int(prev_offset), _ptr(mu), _ptr(token_seq), _ptr(cu_tokens), _ptr(seq_slots), _ptr(out),
+                  N, W, M, dtype_code(x.dtype))
+        return out
+
+    WKV_PIECE = 64  # tokens of one request that are walked in a row before the walk is cut into pieces
+    WKV_MAX_DIM = 128
+
+    def wkv_scan(self, r, k, v, wraw, w0, u, g, norm_w, eps: float, x, state, heads: int, dim: int, seq_slots,
+                 cu_tokens, out_dtype, max_q_len: int = 0) -> torch.Tensor:
+        """Per head, with the matrix state S [dim, dim] of the request (float32, `state[slot, : heads dim dim]`):
+            o_t = (S + diag(u) k_t v_t^T)^T r_t;   S <- diag(exp(-exp(wraw_t + w0))) S + k_t v_t^T
+        and the result [N, heads * dim] in `out_dtype` is o_t / rms(o_t) (per head, eps inside the root)
+        * norm_w * silu(g_t).  r, k, v, wraw float32 [N, heads * dim]; w0, u float32 [heads * dim]; g, x in
+        `out_dtype`.  The last row of every request's x [N, W] is saved behind the matrix state.
+        `max_q_len` (a host-side bound) only decides into how many pieces a walk is cut."""
+        HD = heads * dim
+        for t, name in ((r, "r"), (k, "k"), (v, "v"), (wraw, "wraw"), (w0, "w0"), (u, "u"), (state, "state")):
+            _dev(t, name, torch.float32)
+        _dev(g, "g", out_dtype)
+        _dev(x, "x", out_dtype)
+        _dev(norm_w, "norm weight")
+        _dev(seq_slots, "seq_slots", torch.int32)
+        _dev(cu_tokens, "cu_tokens", torch.int32)
+        N, W = x.shape
+        S = seq_slots.shape[0]
+        _need(0 < dim <= self.WKV_MAX_DIM, f"a head of the recurrence holds at most {self.WKV_MAX_DIM} channels")
+        for t in (r, k, v, wraw, g):
+            _need(t.shape == (N, HD), "r, k, v, wraw and g must be [N, heads * dim]")
+        _need(w0.shape == (HD,) and u.shape == (HD,) and norm_w.shape == (HD,), "w0, u and the norm weight must be [heads * dim]")
+        _need(state.dim() == 2 and state.shape[1] >= HD * dim + W, "a state row holds heads * dim * dim + W floats")
+        _need(cu_tokens.shape == (S + 1,), "cu_tokens must be [S + 1]")
+        out = torch.empty((N, HD), dtype=out_dtype, device=x.device)
+        piece = self.WKV_PIECE
+        pieces = -(-max_q_len // piece) if max_q_len > 2 * piece else 1
+        part = None
+        if pieces > 1:
+            part = torch.empty((S * pieces * heads * (dim * dim + dim),), dtype=torch.float32, device=x.device)
+        else:
+            piece = 1 << 30
+        self._run("wkv", "lle_wkv_scan",
+                  [_P, _P, _P, _P, _P, _P, _P, _P, _I, _F, _P, _P, _L, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
+                  _ptr(r), _ptr(k), _ptr(v), _ptr(wraw), _ptr(w0), _ptr(u), _ptr(g), _ptr(norm_w),
+                  dtype_code(norm_w.dtype), float(eps), _ptr(x), _ptr(state), state.stride(0), HD * dim, _ptr(seq_slots),
+                  _ptr(cu_tokens), _ptr(out), S, heads, dim, W, pieces, piece, _ptr(part), dtype_code(out_dtype))
         return out
 
     # -- picking tokens --------------------------------------------------------------

@@ -410,3 +410,95 @@ extern "C" int lle_qk_norm_rope_write(const void* qkv, const void* slots,
             (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride, write_kv);
     LLE_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------
+// Projections normed as a whole.  A row of `qkv` holds q [nq dim], then (with keys and values of
+// its own) k [nkv dim] and v [nkv vdim], then `extra` columns that are left alone; `bias` (or none)
+// covers the whole row.  q and k are divided by the root mean square of their WHOLE projection
+// (all heads at once), times a weight per element, then the first `rot` elements of every head are
+// rotated in the half-split layout.  The cache's heads hold D >= max(dim, vdim) elements: q leaves
+// as [N, nq, D] and K, V^T go to the pages with zeros past dim and vdim.  grid = tokens.
+// ---------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float pn_value(const T* __restrict__ row, const T* __restrict__ bias, int e) {
+    return to_f32<T>(row[e]) + (bias ? to_f32<T>(bias[e]) : 0.f);
+}
+
+// element e (< dim) of head `head` of a projection that starts at column `col0`, normed and rotated
+template <typename T>
+__device__ __forceinline__ float pn_normed_rotated(const T* __restrict__ row, const T* __restrict__ bias, int col0,
+                                                   int head, int dim, int e, float inv, const void* __restrict__ weight,
+                                                   int wd, const float* __restrict__ cs, int rot) {
+    const int at = head * dim + e;
+    const float x = pn_value<T>(row, bias, col0 + at) * inv * load_as_f32(weight, at, wd);
+    if (e >= rot) return x;
+    const int half = rot / 2;
+    const bool low = e < half;
+    const int i = low ? e : e - half;
+    const int pe = low ? e + half : e - half;
+    const float y = pn_value<T>(row, bias, col0 + head * dim + pe) * inv * load_as_f32(weight, head * dim + pe, wd);
+    const float c = cs[2 * i], s = cs[2 * i + 1];
+    return low ? x * c - y * s : x * c + y * s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void proj_norm_rope_write_kernel(
+    const T* __restrict__ qkv, int cols, const T* __restrict__ bias, const int32_t* __restrict__ slots,
+    const void* __restrict__ q_weight, const void* __restrict__ k_weight, int wd, const float* __restrict__ cos_sin,
+    int rot, float eps, T* __restrict__ q_out, T* __restrict__ kv_layer, int nq, int nkv, int dim, int vdim, int D,
+    int page_size, int64_t page_stride, int has_kv, int write_kv) {
+    __shared__ float red[16];
+    const int64_t n = blockIdx.x;
+    const T* row = qkv + n * cols;
+    const float* cs = cos_sin + n * rot;  // [rot / 2][2]
+    const int qw = nq * dim, kw = nkv * dim;
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < qw; e += blockDim.x) {
+        const float x = pn_value<T>(row, bias, e);
+        ss += x * x;
+    }
+    const float inv_q = 1.0f / sqrtf(block_sum(ss, red) / (float)qw + eps);
+    for (int idx = threadIdx.x; idx < nq * D; idx += blockDim.x) {
+        const int h = idx / D, e = idx - h * D;
+        const float y = e < dim ? pn_normed_rotated<T>(row, bias, 0, h, dim, e, inv_q, q_weight, wd, cs, rot) : 0.f;
+        q_out[n * nq * D + idx] = from_f32<T>(y);
+    }
+    if (!has_kv) return;
+    ss = 0.f;
+    for (int e = threadIdx.x; e < kw; e += blockDim.x) {
+        const float x = pn_value<T>(row, bias, qw + e);
+        ss += x * x;
+    }
+    const float inv_k = 1.0f / sqrtf(block_sum(ss, red) / (float)kw + eps);
+    const int slot = slots[n];
+    if (!write_kv || slot < 0) return;
+    const int page = slot / page_size, off = slot - page * page_size;
+    T* dst = kv_layer + (int64_t)page * page_stride;
+    for (int idx = threadIdx.x; idx < nkv * D; idx += blockDim.x) {
+        const int h = idx / D, e = idx - h * D;
+        const float y = e < dim ? pn_normed_rotated<T>(row, bias, qw, h, dim, e, inv_k, k_weight, wd, cs, rot) : 0.f;
+        dst[((int64_t)h * page_size + off) * D + e] = from_f32<T>(y);
+        const float v = e < vdim ? pn_value<T>(row, bias, qw + kw + h * vdim + e) : 0.f;
+        dst[(int64_t)nkv * page_size * D + ((int64_t)h * D + e) * page_size + off] = from_f32<T>(v);
+    }
+}
+
+extern "C" int lle_proj_norm_rope_write(const void* qkv, int cols, const void* bias, const void* slots,
+                                        const void* q_weight, const void* k_weight, int weight_dtype, const void* cos_sin,
+                                        int rot, float eps, void* q_out, void* kv_layer, int N, int nq, int nkv, int dim,
+                                        int vdim, int D, int page_size, int64_t page_stride, int has_kv, int write_kv,
+                                        int dtype, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (rot % 2 || rot > dim || dim > D || vdim > D || (rot > 0 && cos_sin == nullptr)) return (int)hipErrorInvalidValue;
+    if (dtype == LLE_F32)
+        proj_norm_rope_write_kernel<float><<<N, 256, 0, stream>>>(
+            (const float*)qkv, cols, (const float*)bias, (const int32_t*)slots, q_weight, k_weight, weight_dtype,
+            (const float*)cos_sin, rot, eps, (float*)q_out, (float*)kv_layer, nq, nkv, dim, vdim, D, page_size, page_stride,
+            has_kv, write_kv);
+    else
+        proj_norm_rope_write_kernel<bf16_t><<<N, 256, 0, stream>>>(
+            (const bf16_t*)qkv, cols, (const bf16_t*)bias, (const int32_t*)slots, q_weight, k_weight, weight_dtype,
+            (const float*)cos_sin, rot, eps, (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, dim, vdim, D, page_size,
+            page_stride, has_kv, write_kv);
+    LLE_RETURN_LAUNCH_STATUS();
+}

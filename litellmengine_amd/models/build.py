@@ -8,7 +8,7 @@ import torch
 from ..config.registry import Architecture, architecture_of, get_architecture
 from ..config.model_config import read_config_json
 from ..parts.base import BuildContext
-from ..weights.loader import load_checkpoint
+from ..weights.loader import checkpoint_header, load_checkpoint
 from ..weights.random_init import random_weights
 from ..weights.spec import TensorSpec
 
@@ -46,6 +46,8 @@ def load_model(model_dir: str, dtype, device=None, ops=None):
     d = read_config_json(model_dir)
     arch = architecture_of(d)
     config = arch.config_class.from_dict(d)
+    if hasattr(config, "with_tensor_shapes"):  # sizes that config.json leaves to the checkpoint's shapes
+        config = config.with_tensor_shapes({name: shape for name, (_, shape, _) in checkpoint_header(model_dir).items()})
     model = arch.build(config)
     ctx = make_context(dtype, device, ops)
     weights = load_checkpoint(model_dir, model.tensor_specs(), ctx.dtype, ctx.device)

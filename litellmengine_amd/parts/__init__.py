@@ -1,19 +1,20 @@
-from .attention import PagedAttention
+from .attention import PagedAttention, SinkAttention
 from .base import (Block, BuildContext, CacheField, Carried, CacheSpec, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part,
-                   Normed, PartialSums, PositionEncoding, Prenormed, StateSpec)
-from .block import PostNormBlock, PreNormBlock
+                   Normed, PartialSums, PositionEncoding, Prenormed, ScaledSum, StateSpec)
+from .block import ParallelBlock, PostNormBlock, PreNormBlock
 from .embedding import Embedding
 from .feed_forward import GatedMLP
 from .latent_attention import LatentAttention
 from .linear import Linear
-from .moe import RoutedMLP
+from .moe import GroupLimitedMLP, RoutedMLP
 from .norm import RMSNorm
 from .position import NoPositionEncoding, RotaryHalfSplit, RotaryInterleaved
 from .recurrent import MinGRU
+from .wkv import WKVMixer
 
 __all__ = [
     "Block", "BuildContext", "CacheField", "CacheSpec", "Carried", "LatentAttention", "MinGRU", "PostNormBlock",
     "RoutedMLP", "RotaryInterleaved", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
     "NoPositionEncoding", "Norm", "NormFold", "Normed", "PagedAttention", "Part", "PartialSums", "PositionEncoding", "PreNormBlock", "Prenormed", "RMSNorm",
-    "RotaryHalfSplit", "StateSpec",
+    "RotaryHalfSplit", "StateSpec", "GroupLimitedMLP", "ParallelBlock", "ScaledSum", "SinkAttention", "WKVMixer",
 ]

@@ -19,7 +19,7 @@ from typing import Dict, Optional, Sequence
 import torch
 
 from ..csrc.limits import check_head_dim
-from ..weights.spec import INIT_NORM, TensorSpec
+from ..weights.spec import INIT_NORM, INIT_NORMAL, TensorSpec
 from .base import BuildContext, CacheSpec, KVCacheSpec, Mixer, PositionEncoding
 from .linear import Linear
 
@@ -141,3 +141,102 @@ class PagedAttention(Mixer):
             self.window, self.scale, step.min_q_len, step.max_q_len, step.max_kv_len,
         )
         return self.o.forward(a, fold=fold)
+
+
+class SinkAttention(Mixer):
+    """Grouped-query attention over the paged cache whose softmax has a sink and whose heads are gated:
+
+        q = W_q h + b_q, k = W_k h + b_k, v = W_v h + b_v
+        q, k <- divided by the root mean square of the WHOLE projection (all heads at once), times a
+                weight per element; then the position encoding on the first elements of every head
+        p_j = exp(s_j) / (exp(sink) + sum_j exp(s_j)),  s_j = (q . k_j) * scale,  over the last `window` keys
+        out = W_o [heads' (sum_j p_j v_j) * sigmoid(W_g h)_head]
+
+    Keys may be `dim` wide and values `vdim`: the cache's heads hold `cache_dim` >= both elements (a
+    multiple of 32, which the matrix-core kernels take), the rest zeros, so the kernels of
+    `PagedAttention` serve.  With `own_kv=False` the mixer has no key and value tensors: its plan
+    entry reads the cache that another layer's mixer writes, with queries, window and gate of its
+    own.  `cache_window` is what the cache keeps (the largest window of all mixers that read it;
+    default: this mixer's own)."""
+
+    graph_safe = True
+    UNBOUNDED = object()  # cache_window: keep every position, whatever this mixer's own window
+
+    def __init__(self, prefix: str, hidden_size: int, num_q_heads: int, num_kv_heads: int, dim: int, vdim: int,
+                 position: PositionEncoding, norm_eps: float, scale: float, window: Optional[int] = None,
+                 sink: Optional[float] = 0.0, own_kv: bool = True, cache_window=None,
+                 names: Sequence[str] = ("q", "k", "v", "g", "o"), bias_suffix: str = ".b", norm_suffix: str = ".norm"):
+        if num_q_heads % num_kv_heads:
+            raise ValueError("num_q_heads must be a multiple of num_kv_heads")
+        self.cache_dim = -(-max(dim, vdim) // 32) * 32
+        check_head_dim(self.cache_dim, getattr(position, "rotary_dim", 0))
+        if getattr(position, "rotary_dim", 0) > dim:
+            raise ValueError("the rotation covers more elements than a key has")
+        self.prefix = prefix
+        self.hidden = hidden_size
+        self.nq, self.nkv, self.dim, self.vdim = num_q_heads, num_kv_heads, dim, vdim
+        self.position = position
+        self.eps = float(norm_eps)
+        self.scale = float(scale)
+        self.window = window
+        self.sink = sink
+        self.own_kv = bool(own_kv)
+        if cache_window is SinkAttention.UNBOUNDED:
+            self._cache_window = None
+        else:
+            self._cache_window = window if cache_window is None else cache_window
+        q, k, v, g, o = (prefix + n for n in names)
+        self.q_name, self.k_name, self.v_name, self.g_name = q, k, v, g
+        self.bias_suffix, self.norm_suffix = bias_suffix, norm_suffix
+        self.o = Linear([o], num_q_heads * vdim, [hidden_size])
+        self.weight = self.bias = self.q_norm_w = self.k_norm_w = self.sinks = None
+
+    def _widths(self):
+        w = [(self.q_name, self.nq * self.dim, True)]
+        if self.own_kv:
+            w += [(self.k_name, self.nkv * self.dim, True), (self.v_name, self.nkv * self.vdim, True)]
+        return w + [(self.g_name, self.nq, False)]  # (name, rows, has a bias)
+
+    def cache_spec(self) -> CacheSpec:
+        return KVCacheSpec(self.nkv, self.cache_dim, self._cache_window)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = dict(self.o.tensor_specs())
+        for name, rows, biased in self._widths():
+            specs[name] = TensorSpec((rows, self.hidden), INIT_NORMAL)
+            if biased:
+                specs[name + self.bias_suffix] = TensorSpec((rows,), INIT_NORMAL)
+        specs[self.q_name + self.norm_suffix] = TensorSpec((self.nq * self.dim,), INIT_NORM)
+        if self.own_kv:
+            specs[self.k_name + self.norm_suffix] = TensorSpec((self.nkv * self.dim,), INIT_NORM)
+        return specs
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        self.o.bind(weights, ctx)
+        self.position.bind(weights, ctx)
+        # one product for q, (k, v,) and the gates' inputs; the gates have no bias
+        self.weight = torch.cat([weights[name].to(ctx.dtype) for name, _, _ in self._widths()], dim=0).contiguous()
+        self.bias = torch.cat([
+            weights[name + self.bias_suffix].to(ctx.dtype).reshape(-1) if biased
+            else torch.zeros(rows, dtype=ctx.dtype, device=ctx.device)
+            for name, rows, biased in self._widths()]).contiguous()
+        self.q_norm_w = weights[self.q_name + self.norm_suffix].float().contiguous()
+        self.k_norm_w = weights[self.k_name + self.norm_suffix].float().contiguous() if self.own_kv else None
+        self.sinks = None if self.sink is None else torch.full((self.nq,), float(self.sink), dtype=torch.float32,
+                                                               device=ctx.device)
+
+    def forward(self, x, step, cache):
+        ops = self.ctx.ops
+        if cache.writes != self.own_kv:
+            raise ValueError("a mixer with keys and values of its own writes its cache, one without reads another's")
+        group = cache.group
+        qkvg = ops.linear(x, self.weight)
+        cos_sin, rot = self.position.fused_rotary(step)
+        q = ops.proj_norm_rope_write(qkvg, self.bias, group.slot_mapping, self.q_norm_w, self.k_norm_w, cos_sin, rot,
+                                     self.eps, cache.kv, self.nq, self.nkv, self.dim, self.vdim, self.own_kv, cache.writes)
+        a = ops.paged_attention(q, cache.kv, group.block_table, step.seq_slots, step.cu_tokens, step.kv_lens,
+                                step.token_seq, self.window, self.scale, step.min_q_len, step.max_q_len, step.max_kv_len,
+                                sinks=self.sinks)
+        gated = ops.head_gate(a, qkvg, qkvg.shape[1] - self.nq, self.nq, self.vdim)
+        return self.o.forward(gated)

@@ -165,12 +165,28 @@ class PartialSums:
         return self.sums.sum(0)
 
 
+@dataclasses.dataclass
+class ScaledSum:
+    """What a block whose sublayers run side by side leaves to be added to the residual stream:
+    `mult * (a + b)` (`b` may be None; a, b [N, width], each in the activation type or in 32-bit).
+    Norm.forward takes it where it takes a delta; `total()` is the plain way to take it."""
+
+    a: torch.Tensor
+    b: Optional[torch.Tensor]
+    mult: float
+
+    def total(self) -> torch.Tensor:
+        t = self.a.float() if self.b is None else self.a.float() + self.b.float()
+        return t * self.mult
+
+
 class Norm(Part):
     """forward(hidden, delta) adds `delta` (or nothing) into the 32-bit residual
     stream `hidden` in place and returns the normed rows in the activation type;
     with `rows` only those rows are read and `hidden` is left alone.  `delta` is
     [N, hidden] in the activation type, or the PartialSums that a Linear made with
-    `to_residual` may leave (`delta.total()` is the plain way to take them).
+    `to_residual` may leave, or the ScaledSum of a block whose sublayers run side by
+    side (`delta.total()` is the plain way to take either).
 
     fold(hidden) may return a NormFold when the step is small enough that the
     products on both sides of the norm can do its work (None: call forward).

@@ -8,7 +8,7 @@ from typing import Dict
 from ..weights.spec import TensorSpec
 from typing import Optional
 
-from .base import Block, BuildContext, Carried, FeedForward, Mixer, Norm, Normed, Prenormed
+from .base import Block, BuildContext, Carried, FeedForward, Mixer, Norm, Normed, Prenormed, ScaledSum
 
 
 class PreNormBlock(Block):
@@ -106,3 +106,44 @@ class PostNormBlock(Block):
                 y, extra = y
             x = self.norm_ff.add_normed(hidden, y, extra)
         return Carried(x)
+
+
+class ParallelBlock(Block):
+    """Residual block whose sublayers run side by side on ONE norm's result:
+        h = norm(x);  x <- x + mult * (mixer(h) + ff(h))
+    The sum is left to whoever comes next as a `ScaledSum`: the next norm's kernel adds it into
+    the 32-bit stream, times `mult`, and norms in the same launch.  A block without a
+    feed-forward adds the mixer's result alone."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, feed_forward: Optional[FeedForward] = None, mult: float = 1.0):
+        self.norm = norm
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mult = float(mult)
+
+    def _parts(self):
+        return tuple(p for p in (self.norm, self.mixer, self.feed_forward) if p is not None)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs: Dict[str, TensorSpec] = {}
+        for p in self._parts():
+            specs.update(p.tensor_specs())
+        return specs
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        for p in self._parts():
+            p.bind(weights, ctx)
+
+    def input_norm(self):
+        return self.norm
+
+    def forward(self, hidden, delta, step, cache, next_norm=None):
+        if isinstance(delta, Carried):  # the block before has added everything into the stream itself
+            delta = None
+        if isinstance(delta, Prenormed):
+            raise ValueError("a block of side-by-side sublayers takes no folded norm")
+        h = delta.x if isinstance(delta, Normed) else self.norm.forward(hidden, delta)
+        a = self.mixer.forward(h, step, cache)
+        b = self.feed_forward.forward(h) if self.feed_forward is not None else None
+        return ScaledSum(a, b, self.mult)

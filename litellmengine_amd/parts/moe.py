@@ -69,3 +69,57 @@ class RoutedMLP(FeedForward):
         if self.shared is None:
             return routed
         return routed, self.shared.forward(x)
+
+
+class GroupLimitedMLP(FeedForward):
+    """Mixture of experts whose router scores ALL experts with one softmax and limits its choice to groups:
+
+        s = softmax(W_router h)                        32-bit, over experts and identity experts alike
+        c = s + correction                             the choice scores; the gains never see the correction
+        the experts form `groups` equal groups of neighbours; a group's score is its largest c, and only
+        the experts of the `groups_kept` best groups can be chosen (the others count as minus infinity)
+        chosen = the `top` largest c among those;  gains = s[chosen] / (sum of s[chosen] + 1e-20)
+        out = sum_k gains_k * expert_k(h),  expert(h) = down(silu(gate h) * (up h))
+
+    The last `identity` router outputs are identity experts: no tensors, their result is h itself.  The
+    experts' weights are stacked, the choice stays on the device, the sum is left in 32-bit."""
+
+    def __init__(self, prefix: str, hidden_size: int, expert_size: int, num_experts: int, top: int, identity: int = 0,
+                 groups: int = 1, groups_kept: int = 1, expert_prefix: str = "e{}.", names=("gate", "up", "down"),
+                 router_names=("router", "correction")):
+        total = num_experts + identity
+        if num_experts <= 0 or identity < 0 or groups <= 0 or total % groups or not 0 < groups_kept <= groups:
+            raise ValueError("experts and identity experts together form equal groups, of which some are kept")
+        if not 0 < top <= groups_kept * (total // groups):
+            raise ValueError("every token uses between one and all of the experts of the kept groups")
+        self.prefix, self.hidden, self.ff, self.E, self.identity, self.top = (prefix, hidden_size, expert_size,
+                                                                             num_experts, identity, top)
+        self.groups, self.groups_kept = groups, groups_kept
+        self.expert_names = [[prefix + expert_prefix.format(e) + n for n in names] for e in range(num_experts)]
+        self.router = Linear([prefix + router_names[0]], hidden_size, [total])
+        self.correction_name = prefix + router_names[1]
+        self.correction = self.gate_up = self.down = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = dict(self.router.tensor_specs())
+        specs[self.correction_name] = TensorSpec((self.E + self.identity,), INIT_NORMAL)
+        for gate, up, down in self.expert_names:
+            specs[gate] = TensorSpec((self.ff, self.hidden), INIT_NORMAL)
+            specs[up] = TensorSpec((self.ff, self.hidden), INIT_NORMAL)
+            specs[down] = TensorSpec((self.hidden, self.ff), INIT_NORMAL)
+        return specs
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        self.router.bind(weights, ctx)
+        self.correction = weights[self.correction_name].float().contiguous()
+        self.gate_up = torch.stack(
+            [torch.cat([weights[g].to(ctx.dtype), weights[u].to(ctx.dtype)], dim=0) for g, u, _ in self.expert_names]
+        ).contiguous()
+        self.down = torch.stack([weights[d].to(ctx.dtype) for _, _, d in self.expert_names]).contiguous()
+
+    def forward(self, x):
+        ops = self.ctx.ops
+        logits = self.router.forward(x, out_dtype=torch.float32)
+        ids, gains = ops.moe_route_grouped(logits, self.correction, self.top, self.groups, self.groups_kept)
+        return ops.moe_experts(x, ids, gains, self.gate_up, self.down)  # float32 [N, hidden]; ids from E on: x itself

@@ -7,14 +7,16 @@ from typing import Dict, Optional
 
 import torch
 
-from ..weights.spec import INIT_NORM, TensorSpec
-from .base import BuildContext, Norm, NormFold
+from ..weights.spec import INIT_NORM, INIT_NORMAL, TensorSpec
+from .base import BuildContext, Norm, NormFold, ScaledSum
 
 
 class RMSNorm(Norm):
-    def __init__(self, name: str, size: int, eps: float, scalar: bool = False):
+    def __init__(self, name: str, size: int, eps: float, scalar: bool = False, one_plus: bool = False):
         """`scalar`: the checkpoint holds ONE gain for all coordinates (a tensor without
-        dimensions); the kernels see it repeated `size` times."""
+        dimensions); the kernels see it repeated `size` times.  `one_plus`: the stored weight
+        lies around zero and the gain is 1 + weight (added in 32-bit, kept in 32-bit)."""
+        self.one_plus = bool(one_plus)
         self.name = name
         self.size = size
         self.eps = float(eps)
@@ -22,17 +24,22 @@ class RMSNorm(Norm):
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.name: TensorSpec(() if self.scalar else (self.size,), INIT_NORM)}
+        return {self.name: TensorSpec(() if self.scalar else (self.size,), INIT_NORMAL if self.one_plus else INIT_NORM)}
 
     def bind(self, weights, ctx: BuildContext) -> None:
         self.ctx = ctx
         w = weights[self.name]  # bfloat16 or float32, as stored
+        if self.one_plus:
+            w = 1.0 + w.float()
         self.weight = (w.reshape(1).expand(self.size) if self.scalar else w).contiguous()
 
     def add_normed(self, hidden, y, extra=None) -> torch.Tensor:
         return self.ctx.ops.rmsnorm_add(hidden, y, self.weight, self.eps, self.ctx.dtype, extra)
 
     def forward(self, hidden, delta, rows=None) -> torch.Tensor:
+        if isinstance(delta, ScaledSum):  # the add, times its constant, and the norm in one launch
+            return self.ctx.ops.scaled_add_rmsnorm(hidden, delta.a, delta.b, delta.mult, self.weight, self.eps,
+                                                   self.ctx.dtype, rows)
         return self.ctx.ops.add_rmsnorm(hidden, delta, self.weight, self.eps, self.ctx.dtype, rows)
 
     def of_embedding(self, ids, table, step=None):
@@ -44,6 +51,8 @@ class RMSNorm(Norm):
         return self.ctx.ops.embedding_rmsnorm(ids, table, self.weight, self.eps)
 
     def fold(self, hidden) -> Optional[NormFold]:
+        if self.one_plus:
+            return None
         if not self.ctx.ops.can_fold_norm(hidden.shape[0], self.size, self.ctx.dtype):
             return None
         return NormFold(hidden, self.weight, self.eps)

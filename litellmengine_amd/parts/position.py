@@ -1,11 +1,22 @@
 """Position encodings applied to q and k inside a mixer."""
 from __future__ import annotations
 
+import math
 from typing import Optional
 
 import torch
 
 from .base import BuildContext, PositionEncoding
+
+
+def scaled_frequencies(inv_freq: torch.Tensor, scaling) -> torch.Tensor:
+    """float64 frequencies with their long wavelengths stretched (see RotaryHalfSplit)."""
+    factor, low, high, original = float(scaling.factor), float(scaling.low), float(scaling.high), float(scaling.original)
+    wavelength = 2.0 * math.pi / inv_freq
+    share = (original / wavelength - low) / (high - low)
+    mixed = (1.0 - share) * inv_freq / factor + share * inv_freq
+    out = torch.where(wavelength > original / low, inv_freq / factor, mixed)
+    return torch.where(wavelength < original / high, inv_freq, out)
 
 
 class RotaryHalfSplit(PositionEncoding):
@@ -18,7 +29,12 @@ class RotaryHalfSplit(PositionEncoding):
     the angle, sine and cosine are float32 in the kernel, computed once per step for
     all heads and layers."""
 
-    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None):
+    def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None, scaling=None):
+        """`scaling` (an object with `factor`, `low`, `high`, `original`, or None) stretches long
+        wavelengths: with l = 2 pi / f a frequency is kept where l < original / high, divided by
+        `factor` where l > original / low, and in between it is (1 - s) f / factor + s f with
+        s = (original / l - low) / (high - low)."""
+        self.scaling = scaling
         self.head_dim = head_dim
         self.theta = float(theta)
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
@@ -30,12 +46,18 @@ class RotaryHalfSplit(PositionEncoding):
         self.ctx = ctx
         i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
         inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -(2.0 * i) / self.rotary_dim)
+        if self.scaling is not None:
+            inv = scaled_frequencies(inv, self.scaling)
         self.inv_freq = inv.to(torch.float32).to(ctx.device)
+
+    def _scaling_key(self):
+        s = self.scaling
+        return None if s is None else (float(s.factor), float(s.low), float(s.high), float(s.original))
 
     def fused_rotary(self, step):
         # cosines and sines of this step's positions: made by the first layer that asks,
         # shared by every layer with the same rotation
-        key = ("rope_table", self.theta, self.rotary_dim)
+        key = ("rope_table", self.theta, self.rotary_dim, self._scaling_key())
         table = step.scratch.get(key)
         if table is None:
             table = self.ctx.ops.rope_table(step.positions, self.inv_freq)

@@ -115,7 +115,7 @@ class TorchOps:
         return q.to(qkv.dtype).contiguous()
 
     def paged_attention(self, q, kv_layer, block_table, seq_slots, cu_tokens, kv_lens, token_seq, window, scale,
-                        min_q_len=0, max_q_len=0, max_kv_len=0):
+                        min_q_len=0, max_q_len=0, max_kv_len=0, sinks=None):
         N, nq, d = q.shape
         nkv, P = kv_layer.shape[2], kv_layer.shape[3]
         group = nq // nkv
@@ -136,7 +136,13 @@ class TorchOps:
                 keys = keys.repeat_interleave(group, dim=1)
                 vals = vals.repeat_interleave(group, dim=1)
                 sc = torch.einsum("hd,nhd->hn", q[t].to(self.cd), keys) * scale
-                p = torch.softmax(sc, dim=-1)
+                if sinks is None:
+                    p = torch.softmax(sc, dim=-1)
+                else:  # one more place in every head's sum, with a score of its own and no value
+                    sk = sinks.to(self.cd)[:, None]
+                    big = torch.maximum(sc.max(dim=1, keepdim=True).values, sk)
+                    e = torch.exp(sc - big)
+                    p = e / (e.sum(1, keepdim=True) + torch.exp(sk - big))
                 out[t] = torch.einsum("hn,nhd->hd", p, vals)
         return out.reshape(N, nq * d).to(q.dtype)
 
@@ -262,6 +268,20 @@ class TorchOps:
         vals, idx = torch.topk(v, top, dim=-1)
         return idx.to(torch.int32), torch.softmax(vals, dim=-1).to(torch.float32)
 
+    def moe_route_grouped(self, logits, correction, top, groups=1, keep=1):
+        s = torch.softmax(logits.to(self.cd), dim=-1)
+        c = s + correction.to(self.cd)
+        N, E = c.shape
+        size = E // groups
+        best = c.view(N, groups, size).max(dim=-1).values
+        # (a stable sort: among equal scores the lower index comes first, for groups and for experts)
+        kept = torch.sort(best, dim=-1, descending=True, stable=True).indices[:, :keep]
+        allowed = torch.zeros((N, groups), dtype=torch.bool, device=c.device).scatter_(1, kept, True)
+        c = torch.where(allowed[:, :, None].expand(N, groups, size).reshape(N, E), c, torch.full_like(c, -math.inf))
+        ids = torch.sort(c, dim=-1, descending=True, stable=True).indices[:, :top]
+        chosen = torch.gather(s, 1, ids)
+        return ids.to(torch.int32), (chosen / (chosen.sum(-1, keepdim=True) + 1e-20)).to(torch.float32)
+
     def moe_experts(self, x, ids, gains, gate_up, down):
         N, top = ids.shape
         ff = gate_up.shape[1] // 2
@@ -270,11 +290,108 @@ class TorchOps:
         for n in range(N):
             for k in range(top):
                 e = int(ids[n, k])
+                if e >= gate_up.shape[0]:  # an identity expert
+                    out[n] += gains[n, k].to(self.cd) * xx[n]
+                    continue
                 gu = gate_up[e].to(self.cd) @ xx[n]
                 a = gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]
                 a = a.to(x.dtype).to(self.cd)
                 out[n] += gains[n, k].to(self.cd) * (down[e].to(self.cd) @ a)
         return out.to(torch.float32)
+
+    # -- projections normed as a whole, gates per head, side-by-side sublayers -------------------
+    def proj_norm_rope_write(self, qkv, bias, slots, q_weight, k_weight, cos_sin, rotary_dim, eps, kv_layer,
+                             num_q_heads, num_kv_heads, dim, vdim, has_kv=True, write_kv=True):
+        nq, nkv = num_q_heads, num_kv_heads
+        N = qkv.shape[0]
+        D, P = kv_layer.shape[4], kv_layer.shape[3]
+        x = qkv.to(self.cd)
+        if bias is not None:
+            x = x + bias.to(self.cd)
+
+        def norm(t, w):
+            return t / torch.sqrt((t * t).mean(-1, keepdim=True) + eps) * w.to(self.cd)
+
+        def rope(t):
+            if rotary_dim == 0:
+                return t
+            half = rotary_dim // 2
+            c, s = cos_sin[:, None, :, 0].to(self.cd), cos_sin[:, None, :, 1].to(self.cd)
+            x1, x2 = t[..., :half], t[..., half:rotary_dim]
+            return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s, t[..., rotary_dim:]], dim=-1)
+
+        def padded(t):
+            return torch.nn.functional.pad(t, (0, D - t.shape[-1]))
+
+        qw, kw = nq * dim, nkv * dim
+        q = padded(rope(norm(x[:, :qw], q_weight).reshape(N, nq, dim)))
+        if has_kv and write_kv:
+            k = padded(rope(norm(x[:, qw : qw + kw], k_weight).reshape(N, nkv, dim)))
+            v = padded(x[:, qw + kw : qw + kw + nkv * vdim].reshape(N, nkv, vdim))
+            for n in range(N):
+                slot = int(slots[n])
+                if slot < 0:
+                    continue
+                page, off = slot // P, slot % P
+                kv_layer[page, 0, :, off, :] = k[n].to(kv_layer.dtype)
+                v_pages(kv_layer)[page, :, :, off] = v[n].to(kv_layer.dtype)
+        return q.to(qkv.dtype).contiguous()
+
+    def head_gate(self, a, gates, col0, heads, vdim):
+        N = a.shape[0]
+        g = torch.sigmoid(gates[:, col0 : col0 + heads].to(self.cd))
+        return (a.view(N, heads, -1)[:, :, :vdim].to(self.cd) * g[:, :, None]).reshape(N, heads * vdim).to(a.dtype)
+
+    def tanh_(self, x):
+        x.copy_(torch.tanh(x.to(self.cd)).to(x.dtype))
+        return x
+
+    def scaled_add_rmsnorm(self, hidden, a, b, mult, weight, eps, out_dtype, rows=None):
+        d = a.to(torch.float32) if b is None else a.to(torch.float32) + b.to(torch.float32)
+        if rows is None:
+            hidden += mult * d
+            h = hidden
+        else:
+            h = hidden[rows.long()] + mult * d[rows.long()]
+        x = h.to(self.cd)
+        return (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.to(self.cd)).to(out_dtype)
+
+    # -- recurrence with a matrix state ----------------------------------------------------------
+    def shift_mix(self, x, state, prev_offset, mu, token_seq, cu_tokens, seq_slots):
+        N, W = x.shape
+        xx = x.to(self.cd)
+        prev = torch.zeros_like(xx)
+        prev[1:] = xx[:-1]
+        for s in range(seq_slots.shape[0]):
+            q0, q1 = int(cu_tokens[s]), int(cu_tokens[s + 1])
+            if q1 > q0:
+                prev[q0] = state[int(seq_slots[s]), prev_offset : prev_offset + W].to(self.cd)
+        return (xx[None] + (prev - xx)[None] * mu.to(self.cd)[:, None, :]).to(x.dtype)
+
+    def wkv_scan(self, r, k, v, wraw, w0, u, g, norm_w, eps, x, state, heads, dim, seq_slots, cu_tokens, out_dtype,
+                 max_q_len=0):
+        N, W = x.shape
+        HD = heads * dim
+        decay = torch.exp(-torch.exp(wraw.to(self.cd) + w0.to(self.cd))).view(N, heads, dim)
+        rr, kk, vv = (t.to(self.cd).view(N, heads, dim) for t in (r, k, v))
+        uu = u.to(self.cd).view(heads, dim)
+        out = torch.zeros((N, heads, dim), dtype=self.cd, device=x.device)
+        for s in range(seq_slots.shape[0]):
+            slot = int(seq_slots[s])
+            q0, q1 = int(cu_tokens[s]), int(cu_tokens[s + 1])
+            if q1 <= q0:
+                continue
+            S = state[slot, : HD * dim].to(self.cd).view(heads, dim, dim).clone()
+            for t in range(q0, q1):
+                kv = kk[t][:, :, None] * vv[t][:, None, :]
+                out[t] = torch.einsum("hi,hij->hj", rr[t], S + uu[:, :, None] * kv)
+                S = decay[t][:, :, None] * S + kv
+            state[slot, : HD * dim] = S.reshape(-1).to(state.dtype)
+            state[slot, HD * dim : HD * dim + W] = x[q1 - 1].to(state.dtype)
+        out = out / torch.sqrt((out * out).mean(-1, keepdim=True) + eps)
+        gg = g.to(self.cd)
+        y = out.reshape(N, HD) * norm_w.to(self.cd) * (gg * torch.sigmoid(gg))
+        return y.to(out_dtype)
 
     def argmax(self, logits, scatter=None):
         out = torch.argmax(logits, dim=-1).to(torch.int32)  # torch returns the first maximum
