@@ -118,13 +118,13 @@ def rotate_half(x: torch.Tensor, positions: Sequence[int], freqs: Sequence[float
     2 len(freqs) on pass unchanged."""
     y = x.clone()
     half = len(freqs)
-    for t in range(x.shape[0]):
-        for i, f in enumerate(freqs):
-            ang = float(positions[t]) * f
-            c, s = math.cos(ang), math.sin(ang)
-            a, b = x[t, :, i], x[t, :, i + half]
-            y[t, :, i] = a * c - b * s
-            y[t, :, i + half] = b * c + a * s
+    pos = torch.tensor([float(p) for p in positions], dtype=torch.float64)
+    for i, f in enumerate(freqs):
+        ang = pos * f
+        c, s = torch.cos(ang).to(x.dtype)[:, None], torch.sin(ang).to(x.dtype)[:, None]
+        a, b = x[:, :, i], x[:, :, i + half]
+        y[:, :, i] = a * c - b * s
+        y[:, :, i + half] = b * c + a * s
     return y
 
 
@@ -140,12 +140,13 @@ def attention_keys_values(h: torch.Tensor, w, p: str, m: dict, eps: float):
     return k, v.view(T, G, int(m["vdim"]))
 
 
-def sink_softmax(scores: torch.Tensor) -> torch.Tensor:
-    """exp(s_j) / (1 + sum_j exp(s_j)): a softmax with one more place whose score is 0 and
-    whose share is dropped."""
-    big = torch.clamp(scores.max(), min=0.0)
+def sink_softmax(scores: torch.Tensor, seen: torch.Tensor) -> torch.Tensor:
+    """Row by row over the places where `seen`: exp(s_j) / (1 + sum_j exp(s_j)), a softmax with one more
+    place whose score is 0 and whose share is dropped."""
+    scores = scores.masked_fill(~seen, -math.inf)  # (exp(-inf) = 0: what is not seen has no share)
+    big = torch.clamp(scores.max(dim=-1, keepdim=True).values, min=0.0)
     e = torch.exp(scores - big)
-    return e / (torch.exp(-big) + e.sum())
+    return e / (torch.exp(-big) + e.sum(dim=-1, keepdim=True))
 
 
 def attention_mixer(h: torch.Tensor, w, p: str, m: dict, eps: float, keys=None, values=None) -> torch.Tensor:
@@ -158,15 +159,16 @@ def attention_mixer(h: torch.Tensor, w, p: str, m: dict, eps: float, keys=None, 
     q = rms_unit(q, eps) * w[p + "q.norm"]
     freqs = scaled_frequencies(m["rot"]["base"], int(m["rot"]["dims"]), m["rot"].get("scaling"))
     q = rotate_half(q.view(T, H, dim), range(T), freqs)
-    window = int(m["mask"]["size"]) if m.get("mask") else None
+    i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
+    seen = j <= i  # a position sees itself and what came before ...
+    if m.get("mask"):
+        seen = seen & (i - j < int(m["mask"]["size"]))  # ... as far back as the window reaches
     gate = sigmoid(h @ w[p + "g"].T)  # [T, H]
     out = torch.zeros((T, H, vdim), dtype=h.dtype)
     for a in range(H):
         g = a // (H // G)
-        for i in range(T):
-            lo = 0 if window is None else max(0, i - window + 1)
-            s = (keys[lo : i + 1, g] @ q[i, a]) * float(m["scale"])
-            out[i, a] = (sink_softmax(s)[:, None] * values[lo : i + 1, g]).sum(0) * gate[i, a]
+        s = (q[:, a] @ keys[:, g].T) * float(m["scale"])
+        out[:, a] = (sink_softmax(s, seen) @ values[:, g]) * gate[:, a : a + 1]
     return out.reshape(T, H * vdim) @ w[p + "o"].T
 
 

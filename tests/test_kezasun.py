@@ -1,0 +1,369 @@
+"""Kezasun on the CPU: the plain model's mechanisms pinned by their own invariants, the
+configuration and the checkpoint, and the engine (cache, state slots, step function, scheduler,
+trace replay) with substitute kernels against the plain model."""
+import dataclasses
+import math
+import os
+
+import pytest
+import torch
+
+from litellmengine_amd.cache import CacheManager
+from litellmengine_amd.config import ConfigError, KezasunConfig, load_config
+from litellmengine_amd.config.registry import architecture_of
+from litellmengine_amd.engine import LLMEngine, ModelRunner, StepEntry
+from litellmengine_amd.models import load_model
+from litellmengine_amd.parts.position import scaled_frequencies
+from litellmengine_amd.weights.loader import WeightError
+from tests.kezasun_util import CONFIGS, PAGE_SIZES, make_model_dir, plain_logits, rewrite, run_tool, sharpen
+from tests.plain import kezasun_plain as plain
+from tests.tiny import random_tokens
+from tests.torch_ops import TorchOps
+from tests.trace_util import TraceBuilder, changing_portions, check_dumps, mixed, tail_one_by_one, whole
+
+
+def rnd(shape, seed, scale=1.0):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed), dtype=torch.float64) * scale
+
+
+# -- the plain model's mechanisms, each alone ------------------------------------------------
+def test_plain_recurrence_written_out_and_carried_over():
+    T, d = 7, 5
+    r, k, v = rnd((T, d), 1), rnd((T, d), 2), rnd((T, d), 3)
+    decay, u = torch.rand((T, d), generator=torch.Generator().manual_seed(4), dtype=torch.float64), rnd((d,), 5)
+    o, S = plain.wkv_recurrence(r, k, v, decay, u)
+    # the last output written out: past tokens decayed by everything between them and now, the current one with u
+    want = torch.zeros(d, dtype=torch.float64)
+    for j in range(d):
+        for i in range(d):
+            acc = u[i] * k[T - 1, i] * v[T - 1, j]
+            for t in range(T - 1):
+                acc = acc + torch.prod(decay[t + 1 : T - 1, i]) * k[t, i] * v[t, j]
+            want[j] += r[T - 1, i] * acc
+    assert torch.allclose(o[T - 1], want, atol=1e-12)
+    # the second half from the state after the first equals the whole
+    _, S3 = plain.wkv_recurrence(r[:3], k[:3], v[:3], decay[:3], u)
+    o2, S2 = plain.wkv_recurrence(r[3:], k[3:], v[3:], decay[3:], u, state=S3)
+    assert torch.allclose(o2, o[3:], atol=1e-12) and torch.allclose(S2, S, atol=1e-12)
+    # the first token sees nothing but itself, through the bonus
+    assert torch.allclose(o[0], (r[0] * u * k[0]).sum() * v[0], atol=1e-12)
+
+
+def test_plain_decay_lies_between_zero_and_one_and_shift_starts_from_zeros():
+    w = {"m.w1": rnd((3, 6), 1), "m.w2": rnd((8, 3), 2), "m.w0": rnd((8,), 3)}
+    d = plain.wkv_decay(rnd((9, 6), 4), w, "m.")
+    assert d.shape == (9, 8) and float(d.min()) >= 0 and float(d.max()) < 1
+    h = rnd((4, 6), 5)
+    s = plain.token_shift(h)
+    assert torch.equal(s[0], torch.zeros(6, dtype=torch.float64)) and torch.equal(s[1:], h[:-1])
+    assert torch.equal(plain.token_shift(h, first=h[3])[0], h[3])
+
+
+def test_plain_rotation_pairs_halves_and_leaves_the_rest():
+    x = rnd((5, 3, 10), 7)
+    freqs = plain.scaled_frequencies(100.0, 6, None)
+    y = plain.rotate_half(x, [0, 1, 2, 3, 40], freqs)
+    assert torch.equal(y[0], x[0]) and torch.equal(y[..., 6:], x[..., 6:])
+    for i in range(3):  # element i with element i + 3: norms of the pairs stay
+        assert torch.allclose(y[..., i] ** 2 + y[..., i + 3] ** 2, x[..., i] ** 2 + x[..., i + 3] ** 2, atol=1e-12)
+    a = 40 * 100.0 ** (-2 / 6)
+    assert torch.allclose(y[4, :, 1], x[4, :, 1] * math.cos(a) - x[4, :, 4] * math.sin(a), atol=1e-12)
+    # scores depend on the distance of two positions only
+    q, k = rnd((1, 1, 6), 8), rnd((1, 1, 6), 9)
+    dot = lambda p, r: float((plain.rotate_half(q, [p], freqs) * plain.rotate_half(k, [r], freqs)).sum())
+    assert abs(dot(9, 4) - dot(105, 100)) < 1e-9
+
+
+def test_stretched_frequencies_in_three_bands():
+    s = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 1024}
+    plain_f = plain.scaled_frequencies(250000.0, 16, None)
+    got = plain.scaled_frequencies(250000.0, 16, s)
+    bands = set()
+    for f, g in zip(plain_f, got):
+        l = 2 * math.pi / f
+        if l < 256:
+            assert g == f
+            bands.add("short")
+        elif l > 1024:
+            assert g == f / 8.0
+            bands.add("long")
+        else:
+            assert f / 8.0 < g < f
+            bands.add("between")
+    assert bands == {"short", "long", "between"}
+    # the engine's own table, made from the same numbers, agrees
+    cfg = KezasunConfig.from_dict(CONFIGS["B"]).layers[4].mixer
+    i = torch.arange(cfg.rot_dims // 2, dtype=torch.float64)
+    mine = scaled_frequencies(torch.pow(torch.tensor(cfg.rot_base, dtype=torch.float64), -2.0 * i / cfg.rot_dims), cfg.rot_scaling)
+    want = plain.scaled_frequencies(cfg.rot_base, cfg.rot_dims, dataclasses.asdict(cfg.rot_scaling))
+    assert torch.allclose(mine, torch.tensor(want, dtype=torch.float64), rtol=1e-14)
+
+
+def test_plain_sink_takes_weight_and_gives_nothing():
+    seen = torch.ones((1, 4), dtype=torch.bool)
+    p = plain.sink_softmax(torch.zeros((1, 4), dtype=torch.float64), seen)
+    assert torch.allclose(p, torch.full((1, 4), 0.2, dtype=torch.float64))  # four keys and the sink share alike
+    p = plain.sink_softmax(torch.full((1, 4), -50.0, dtype=torch.float64), seen)
+    assert float(p.sum()) < 1e-20  # all keys far below the sink: next to nothing comes through
+    p = plain.sink_softmax(torch.tensor([[800.0, 0.0, 0.0, 0.0]], dtype=torch.float64), seen)
+    assert abs(float(p[0, 0]) - 1.0) < 1e-12  # no overflow
+    half = torch.tensor([[True, True, False, False]])
+    p = plain.sink_softmax(torch.zeros((1, 4), dtype=torch.float64), half)
+    assert torch.allclose(p, torch.tensor([[1 / 3, 1 / 3, 0.0, 0.0]], dtype=torch.float64))
+
+
+def test_plain_window_counts_the_query_itself():
+    """With a window of 3 position 5 sees 3, 4 and 5: the value of key 2 does not matter, that of key 3 does."""
+    m = {"heads": 1, "kv_heads": 1, "dim": 4, "vdim": 4, "scale": 0.5, "mask": {"size": 3}, "rot": {"base": 10.0, "dims": 2}}
+    w = {"a.q": rnd((4, 6), 1), "a.q.b": rnd((4,), 2), "a.k": rnd((4, 6), 3), "a.k.b": rnd((4,), 4), "a.v": rnd((4, 6), 5),
+         "a.v.b": rnd((4,), 6), "a.q.norm": torch.ones(4, dtype=torch.float64), "a.k.norm": torch.ones(4, dtype=torch.float64),
+         "a.g": rnd((1, 6), 7), "a.o": torch.eye(4, dtype=torch.float64)}
+    h = rnd((6, 6), 8)
+    keys, values = plain.attention_keys_values(h, w, "a.", m, 1e-6)
+    base = plain.attention_mixer(h, w, "a.", m, 1e-6, keys, values)
+    v2 = values.clone()
+    v2[2] += 100.0
+    assert torch.equal(plain.attention_mixer(h, w, "a.", m, 1e-6, keys, v2)[5], base[5])
+    v3 = values.clone()
+    v3[3] += 100.0
+    assert not torch.allclose(plain.attention_mixer(h, w, "a.", m, 1e-6, keys, v3)[5], base[5])
+
+
+def test_plain_router_groups_correction_and_identity():
+    z = torch.tensor([2.0, 0.0, 0.1, 0.2, 1.0, 1.1], dtype=torch.float64)
+    zero = torch.zeros(6, dtype=torch.float64)
+    s = torch.softmax(z, 0)
+    ids, gains = plain.router_choice(z, zero, 2, 3, 3)
+    assert ids == [0, 5] and torch.allclose(gains, s[[0, 5]] / s[[0, 5]].sum())
+    # groups (0, 1), (2, 3), (4, 5): only the best group may be chosen from, although expert 5 beats expert 1
+    ids, _ = plain.router_choice(z, zero, 2, 3, 1)
+    assert ids == [0, 1]
+    # the correction moves the choice, never the gains; a negative choice score still beats a group that is left out
+    corr = torch.tensor([-9.0, -9.0, 0.0, 0.0, -9.5, -9.5], dtype=torch.float64)
+    ids, gains = plain.router_choice(z, corr, 3, 3, 2)
+    assert ids == [3, 2, 0] and torch.allclose(gains, s[[3, 2, 0]] / s[[3, 2, 0]].sum())
+    # an identity expert hands its input on
+    w = {"f.router": torch.zeros((3, 4), dtype=torch.float64), "f.correction": torch.tensor([0.0, 5.0, 0.0], dtype=torch.float64),
+         "f.e0.gate": rnd((2, 4), 1), "f.e0.up": rnd((2, 4), 2), "f.e0.down": rnd((4, 2), 3)}
+    h = rnd((3, 4), 4)
+    f = {"router": {"experts": 1, "identity": 2, "top": 1}, "expert": {"ff": 2}}
+    assert torch.allclose(plain.routed_ff(h, w, "f.", f), h)
+
+
+# -- configuration and checkpoint ---------------------------------------------------------------
+@pytest.mark.parametrize("which", list(CONFIGS))
+def test_config_round_trip_and_registry(tmp_path, which):
+    cfg = KezasunConfig.from_dict(CONFIGS[which])
+    assert KezasunConfig.from_dict(cfg.to_dict()) == cfg
+    assert architecture_of(CONFIGS[which]).name == "Kezasun"
+    d = make_model_dir(tmp_path, which)
+    assert load_config(d) == cfg
+    model = load_model(d, "float32", device="cpu", ops=TorchOps())
+    readers = [e for e in model.plan if not e.writes]
+    assert len(readers) == sum(1 for l in CONFIGS[which]["layers"] if l["mixer"].get("kv_from") is not None)
+
+
+def test_sizes_left_to_the_checkpoint_and_defaults(tmp_path):
+    """A config.json that does not say the decay's inner rank: it is the shape of the layer's first decay
+    projection.  Absent keys: no window, no stretching, no identity experts, one group."""
+    import json
+
+    d = make_model_dir(tmp_path, "A")
+    with open(os.path.join(d, "config.json")) as f:
+        raw = json.load(f)
+    for layer in raw["layers"]:
+        layer["mixer"].pop("decay_rank", None)
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(raw, f)
+    cfg = load_config(d)
+    assert [l.mixer.decay_rank for l in cfg.layers if l.type == "wkv"] == [8, 5]
+    load_model(d, "float32", device="cpu", ops=TorchOps())
+    bare = KezasunConfig.from_dict({"architecture": "Kezasun", "vocab": 9, "width": 8, "norm": {"eps": 1e-6}, "layers": [
+        {"type": "attention", "mixer": {"heads": 2, "dim": 4}, "mlp": {"router": {"experts": 3, "top": 2}, "expert": {"ff": 5}}}]})
+    m, f = bare.layers[0].mixer, bare.layers[0].mlp
+    assert (m.kv_heads, m.vdim, m.window, m.rot_dims, m.rot_scaling, m.kv_from) == (2, 4, None, 0, None, None)
+    assert (f.identity, f.groups, f.groups_kept) == (0, 1, 1) and bare.residual_mult == 1.0
+    with pytest.raises(ValueError, match="rank"):
+        from litellmengine_amd.models.kezasun import build_kezasun
+        build_kezasun(KezasunConfig.from_dict(raw))
+
+
+def test_config_faults_are_named():
+    def broken(change):
+        import copy
+        c = copy.deepcopy(CONFIGS["A"])
+        change(c)
+        return c
+
+    cases = [
+        (lambda c: c["layers"][0].update(type="conv"), "type"),
+        (lambda c: c["layers"][0]["mixer"].update(kv_heads=4), "kv_heads"),
+        (lambda c: c["layers"][0]["mixer"]["rot"].update(dims=26), "rot.dims"),
+        (lambda c: c["layers"][2]["mixer"].update(kv_from=1), "kv_from"),
+        (lambda c: c["layers"][2]["mixer"].update(kv_from=4), "kv_from"),
+        (lambda c: c["layers"][2]["mixer"].update(vdim=8), "kv_from"),
+        (lambda c: c["layers"][0]["mlp"]["router"]["groups"].update(count=4), "groups"),
+        (lambda c: c["layers"][0]["mlp"]["router"].update(top=5), "top"),
+        (lambda c: c.pop("norm"), "norm"),
+        (lambda c: c.pop("vocab"), "vocab"),
+    ]
+    for change, word in cases:
+        with pytest.raises(ConfigError, match=word):
+            KezasunConfig.from_dict(broken(change))
+
+
+def test_checkpoint_faults_are_listed_together(tmp_path):
+    from safetensors.torch import load_file, save_file
+
+    d = make_model_dir(tmp_path, "C")
+    path = os.path.join(d, "model.safetensors")
+    t = load_file(path)
+    del t["l3.mlp.e3.up"]
+    t["l0.mix.q.b"] = torch.zeros(4)
+    t["l2.mix.k"] = torch.zeros((8, 48))  # a layer that makes keys of its own has them; l1 (a recurrence) has no such tensor
+    t["l1.norm9"] = torch.zeros(())
+    save_file(t, path)
+    with pytest.raises(WeightError) as e:
+        load_model(d, "float32", device="cpu", ops=TorchOps())
+    assert "l3.mlp.e3.up" in str(e.value) and "l1.norm9" in str(e.value) and "l0.mix.q.b" in str(e.value)
+
+
+def test_a_layer_that_reads_anothers_keys_has_no_key_tensors(tmp_path):
+    d = make_model_dir(tmp_path, "B")
+    model = load_model(d, "float32", device="cpu", ops=TorchOps())
+    names = set(model.tensor_specs())
+    assert "l1.mix.k" in names and "l1.mix.v.b" in names and "l1.mix.k.norm" in names
+    assert not any(n.startswith("l2.mix.k") or n.startswith("l2.mix.v") for n in names)
+    assert {"l2.mix.q", "l2.mix.q.b", "l2.mix.q.norm", "l2.mix.g", "l2.mix.o"} <= names
+    # the cache keeps what the widest reader needs
+    cache = CacheManager(model, page_size=16, num_pages=8, max_requests=2, dtype=torch.float32, device="cpu")
+    assert sorted(str(g.window) for g in cache.groups) == ["48", "None"]
+
+
+# -- the engine with substitute kernels -------------------------------------------------------
+def cpu_runner(d, page_size, num_pages, max_requests=4):
+    model = load_model(d, "float32", device="cpu", ops=TorchOps())
+    cache = CacheManager(model, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
+                         dtype=torch.float32, device="cpu")
+    return model, cache, ModelRunner(model, cache)
+
+
+def watch_layers(model, seen, to=lambda t: t):
+    """After every block: the residual stream with what the block leaves to be added to it."""
+    for b in model.blocks:
+        def wrapped(hidden, delta, step, layer_cache, next_norm=None, inner=b.forward):
+            out = inner(hidden, delta, step, layer_cache, next_norm=next_norm)
+            seen.append(to(hidden.double() + out.total().double()))
+            return out
+        b.forward = wrapped
+
+
+@pytest.mark.parametrize("which", list(CONFIGS))
+def test_one_layer_at_a_time_follows_the_plain_model(tmp_path, which):
+    """The residual stream after every block of a whole prompt."""
+    d = make_model_dir(tmp_path, which)
+    sharpen(d, 8.0)
+    cfg, w = plain.read_model_dir(d)
+    tokens = random_tokens(45, cfg["vocab"], 3)
+    want = plain.residual_streams(tokens, w, cfg)
+    model, cache, runner = cpu_runner(d, PAGE_SIZES[which], 16)
+    seen = []
+    watch_layers(model, seen)
+    runner.step([StepEntry(runner.admit(), tokens, [])])
+    for i, (got, ref) in enumerate(zip(seen, want)):
+        assert (got - ref).abs().max() < 1e-5 * max(1.0, float(ref.abs().max())), f"layer {i} ({cfg['layers'][i]['type']})"
+    for b in model.blocks:
+        del b.forward  # (the wrappers hold the model in a cycle)
+
+
+def all_ways_trace(requests):
+    tb = TraceBuilder()
+    names = list(requests)
+    whole(tb, names[0] + "#whole", requests[names[0]])
+    tail_one_by_one(tb, names[1] + "#tail", requests[names[1]], tail=20)
+    changing_portions(tb, names[2] + "#cut", requests[names[2]], seed=1)
+    mixed(tb, {rid + "#mix": t for rid, t in requests.items()}, seed=5)
+    return tb
+
+
+@pytest.mark.parametrize("which", list(CONFIGS))
+def test_trace_cpu(tmp_path, which):
+    """Whole, with a decoded tail, in portions down to two tokens, and mixed in a pool of the live peak
+    with four slots (pages, slots and state rows are used again)."""
+    d = make_model_dir(tmp_path, which)
+    sharpen(d, 8.0)
+    vocab = CONFIGS[which]["vocab"]
+    requests = {rid: random_tokens(n, vocab, 20 + i) for i, (rid, n) in enumerate(
+        {"a": 70, "b": 45, "c": 100, "d": 33, "e": 64, "f": 1}.items())}
+    tb = all_ways_trace(requests)
+    out = str(tmp_path / "out")
+    run_tool(d, "float32", out, tb, page_size=PAGE_SIZES[which], in_process_ops=TorchOps())
+    check_dumps(out, tb, plain_logits(d, requests), 2e-5)
+
+
+def test_state_rows_are_zeroed_when_a_slot_is_used_again(tmp_path):
+    d = make_model_dir(tmp_path, "A")
+    sharpen(d, 8.0)
+    cfg, w = plain.read_model_dir(d)
+    model, cache, runner = cpu_runner(d, 4, 12, max_requests=1)
+    first, second = random_tokens(9, 131, 1), random_tokens(6, 131, 2)
+    s = runner.admit()
+    runner.step([StepEntry(s, first, [])])
+    assert all(float(st[s].abs().max()) > 0 for st in cache.states.values()) and len(cache.states) == 2
+    runner.release(s)
+    s2 = runner.admit()
+    assert s2 == s and all(float(st[s].abs().max()) == 0 for st in cache.states.values())
+    got = runner.step([StepEntry(s2, second, [5])])
+    assert (got[0].double() - plain.model_logits(second, w, cfg)[5]).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("which", ["A", "C"])
+def test_greedy_generation_through_the_scheduler(tmp_path, which):
+    """Requests of unequal lengths batched, prompts in portions, then a pool so small that requests
+    are preempted and recomputed (their state rows start from zero again): the same tokens."""
+    d = make_model_dir(tmp_path, which)
+    sharpen(d, 8.0)
+    cfg, w = plain.read_model_dir(d)
+    prompts = [random_tokens(n, cfg["vocab"], 40 + i) for i, n in enumerate((1, 7, 23, 40))]
+    want = [plain.generate_greedy(p, w, cfg, 6) for p in prompts]
+    for run_ahead in (False, True):
+        model = load_model(d, "float32", device="cpu", ops=TorchOps())
+        eng = LLMEngine(model, page_size=8, num_pages=16, max_requests=4, prefill_chunk=16, max_tokens_per_step=24,
+                        run_ahead=run_ahead)
+        assert eng.generate(prompts, 6) == want
+    small = LLMEngine(load_model(d, "float32", device="cpu", ops=TorchOps()), page_size=8, num_pages=8, max_requests=4,
+                      prefill_chunk=16, max_tokens_per_step=24, run_ahead=False)
+    assert small.generate(prompts, 6) == want
+    assert all(g.pool.num_held == 0 for g in small.cache.groups)
+
+
+def test_a_lost_key_a_lost_sink_or_a_lost_state_would_show(tmp_path):
+    """The measure of the GPU traces with sharpened weights: in the plain model of such weights, dropping the key
+    at every window's far edge, or the sink, or what the recurrences knew before the last 60 tokens, moves the
+    logits of many positions by far more than the 32-bit tolerance (a peaked softmax has its peak at the window's far
+    edge for one query in so many as the window holds keys)."""
+    d = make_model_dir(tmp_path, "A", seed=5, dtype=torch.bfloat16)
+    sharpen(d, 9.0, fixed_routes=True, memory=1.6)
+    cfg, w = plain.read_model_dir(d)
+    tokens = random_tokens(140, cfg["vocab"], 42)
+    base = plain.model_logits(tokens, w, cfg)
+    narrower = {**cfg, "layers": [dict(l, mixer=dict(l["mixer"], mask={"size": l["mixer"]["mask"]["size"] - 1}))
+                                  if l["mixer"].get("mask") else l for l in cfg["layers"]]}
+    moved = (plain.model_logits(tokens, w, narrower) - base).abs().max(dim=1).values / base.abs().max()
+    assert float((moved[40:] > 1e-3).float().mean()) > 0.25 and float(moved.max()) > 5e-3
+    with_sink = plain.sink_softmax
+    try:  # the softmax without the sink's place
+        plain.sink_softmax = lambda s, seen: torch.softmax(s.masked_fill(~seen, -math.inf), dim=-1)
+        moved = (plain.model_logits(tokens, w, cfg) - base).abs().max(dim=1).values / base.abs().max()
+    finally:
+        plain.sink_softmax = with_sink
+    assert float((moved > 1e-3).float().mean()) > 0.5
+    # recurrences that start anew 60 tokens before the end (a model of the recurrence layers alone)
+    kept = [i for i, l in enumerate(cfg["layers"]) if l["type"] == "wkv"]
+    only = {**cfg, "layers": [cfg["layers"][i] for i in kept]}
+    w2 = {k: v for k, v in w.items() if not k.startswith("l")}
+    for n, i in enumerate(kept):
+        w2.update({f"l{n}." + k[len(f"l{i}."):]: v for k, v in w.items() if k.startswith(f"l{i}.")})
+    whole_run = plain.model_logits(tokens, w2, only)[-1]
+    fresh = plain.model_logits(tokens[-60:], w2, only)[-1]
+    assert float((whole_run - fresh).abs().max() / whole_run.abs().max()) > 1e-3
