@@ -9,6 +9,7 @@
     python bench.py --workload mixed-32b [--layers L]             # a prompt chunk beside 63 decoded tokens
     python bench.py --workload serving                            # requests of many lengths arriving over time
     python bench.py --workload visadra [--sizes small|mid|wide]   # Visadra beside Qwen3 at equal layer sizes, kernel by kernel
+    python bench.py --workload kezasun [--sizes small|mid|wide]   # Kezasun beside Visadra, kernel by kernel
 
 A "step" is one decode step of the whole engine (scheduler, model step over the
 paged cache, sampling) with `batch` live requests whose context ends at
@@ -583,6 +584,185 @@ def visadra_workload(args):
     return 0
 
 
+KEZASUN_SIZES = {
+    # width, wkv heads, wkv dim, decay rank, q heads, kv heads, dim, vdim, rotated, window, experts, identity, top, expert ff, groups, kept
+    "small": (1024, 16, 64, 32, 8, 2, 128, 128, 64, 1024, 16, 4, 4, 512, 4, 2),
+    "mid": (2048, 32, 64, 64, 16, 4, 128, 128, 64, 2048, 64, 8, 6, 1408, 8, 4),
+    "wide": (4096, 64, 64, 64, 32, 8, 128, 128, 64, 4096, 64, 8, 6, 2048, 8, 4),
+}
+
+
+def kezasun_config(which, groups):
+    from litellmengine_amd.config import KezasunConfig
+
+    W, wh, wd, rank, H, G, dim, vdim, rot, window, E, I, top, eff, ng, keep = KEZASUN_SIZES[which]
+    att = {"heads": H, "kv_heads": G, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "mask": {"size": window},
+           "rot": {"base": 250000.0, "dims": rot, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    moe = {"kind": "moe", "expert": {"ff": eff},
+           "router": {"experts": E, "identity": I, "top": top, "groups": {"count": ng, "keep": keep}}}
+    rec = {"heads": wh, "dim": wd, "decay_rank": rank}
+    layers = []
+    for g in range(groups):
+        layers += [{"type": "wkv", "mixer": rec, "mlp": moe}, {"type": "attention", "mixer": att, "mlp": moe},
+                   {"type": "wkv", "mixer": rec, "mlp": moe},
+                   {"type": "attention", "mixer": dict(att, kv_from=4 * g + 1), "mlp": moe}]
+    return KezasunConfig.from_dict({"architecture": "Kezasun", "vocab": 32768, "width": W, "residual_mult": 0.3,
+                                    "norm": {"eps": 1e-6}, "layers": layers})
+
+
+def kezasun_kernels(which):
+    """Each kernel of Kezasun's own at two shapes (a 2048-token prompt; 8 decoded tokens after 4096) beside the
+    like kernel of Visadra (the closest model: a recurrence, attention with a sink, routed experts) at its
+    sizes of the same name: microseconds and the share of its roofline."""
+    import torch
+
+    from litellmengine_amd.csrc.ops import default_ops
+
+    ops = default_ops()
+    W, wh, wd, rank, H, G, dim, vdim, rot, window, E, I, top, eff, ng, keep = KEZASUN_SIZES[which]
+    VW, VH, vdim_k, vrot, vvdim, vrank, gw, vff, VE, vtop, veff, vsff = VISADRA_SIZES[which]
+    dev, bf = "cuda", torch.bfloat16
+    P = PAGE_SIZE
+    rnd = lambda *shape, dtype=bf, scale=1.0: (torch.randn(shape, device=dev) * scale).to(dtype)
+    ints = lambda values: torch.tensor(values, dtype=torch.int32, device=dev)
+    out = {}
+
+    def entry(name, seconds, flops, nbytes, like=None):
+        floor = max(flops / MFMA_PEAK["bf16"], nbytes / HBM_PEAK)
+        e = {"us": round(seconds * 1e6, 1), "roofline_us": round(floor * 1e6, 2), "frac": round(floor / seconds, 4),
+             "bound": "mfma" if flops / MFMA_PEAK["bf16"] > nbytes / HBM_PEAK else "hbm"}
+        if like is not None:
+            e["like"] = like
+            e["times_farther_from_roofline"] = round(like["frac"] / e["frac"], 2) if e["frac"] > 0 else None
+        out[name] = e
+        return e
+
+    for shape, S, q_len, past in (("prefill_2048", 1, 2048, 0), ("decode_b8_ctx4096", 8, 1, 4095)):
+        N, kv = S * q_len, past + q_len
+        pages_each = -(-kv // P)
+        table = torch.arange(S * pages_each, dtype=torch.int32, device=dev).view(S, pages_each).contiguous()
+        seq_slots, cu = ints(list(range(S))), ints([i * q_len for i in range(S + 1)])
+        kv_lens = ints([kv] * S)
+        token_seq = ints([i // q_len for i in range(N)])
+        positions = ints([past + i % q_len for i in range(N)])
+        slots = (table.long().repeat_interleave(P, 1)[:, past:kv] * P + torch.arange(past, kv, device=dev) % P).reshape(-1).int()
+        # attention over a window with a sink beside latent attention with a sink
+        seen = sum(min(window, past + i + 1) for i in range(q_len)) * S  # (query, key) pairs inside the window
+        D = -(-max(dim, vdim) // 32) * 32
+        kv_layer = rnd(S * pages_each + 1, 2, G, P, D)
+        q = rnd(N, H, D, scale=0.1)
+        sinks = torch.zeros(H, device=dev)
+        t = timed_launches(lambda: ops.paged_attention(q, kv_layer, table, seq_slots, cu, kv_lens, token_seq, window, 0.1,
+                                                       q_len, q_len, kv, sinks=sinks))
+        lat_pages = rnd(S * pages_each + 1, P * (2 * vrank + vrot))
+        q_lat, q_rot = rnd(VH, N, vrank, scale=0.1).transpose(0, 1), rnd(N, VH, vrot, dtype=torch.float32, scale=0.1)
+        vsink = torch.zeros(VH, device=dev)
+        tv = timed_launches(lambda: ops.latent_attention(q_lat, q_rot, lat_pages, P, vrank, vrot, table, seq_slots, cu, kv_lens,
+                                                         token_seq, vsink, None, 0.1, q_len, kv, bf))
+        visible = S * (q_len * past + q_len * (q_len + 1) / 2)
+        like = entry(f"{shape}/latent_attention (Visadra)", tv, 2.0 * VH * (2 * vrank + vrot) * visible,
+                     2.0 * (S * kv * (2 * vrank + vrot) + 2 * N * VH * vrank))
+        keys_read = S * min(kv, window + q_len - 1)
+        entry(f"{shape}/paged_attention, window and sink", t, 4.0 * H * D * seen, 2.0 * (keys_read * 2 * G * D + 2 * N * H * D),
+              dict(like, name="latent_attention"))
+        # norm over the whole projection, rotation and the cache write beside the latents' way into the pages
+        cols = H * dim + G * (dim + vdim) + H
+        qkv, bias = rnd(N, cols), rnd(cols)
+        qw, kw = torch.ones(H * dim, device=dev), torch.ones(G * dim, device=dev)
+        cos_sin = ops.rope_table(positions, torch.ones(rot // 2, device=dev))
+        t = timed_launches(lambda: ops.proj_norm_rope_write(qkv, bias, slots, qw, kw, cos_sin, rot, 1e-6, kv_layer, H, G, dim, vdim))
+        dkv, nw = rnd(N, vrank + vrot), torch.ones(vrank, device=dev, dtype=bf)
+        cs2 = ops.rope_table(positions, torch.ones(vrot // 2, device=dev))
+        tv = timed_launches(lambda: ops.latent_kv_write(dkv, nw, 1e-6, cs2, vrot, slots, lat_pages, P, vrank, vrot))
+        like = entry(f"{shape}/latent_kv_write (Visadra)", tv, 0, 2.0 * N * (3 * vrank + 2 * vrot))
+        entry(f"{shape}/proj_norm_rope_write", t, 0, 2.0 * N * (cols + H * D + 2 * G * D), dict(like, name="latent_kv_write"))
+        a = rnd(N, H * D)
+        t = timed_launches(lambda: ops.head_gate(a, qkv, cols - H, H, vdim))
+        entry(f"{shape}/head_gate", t, 0, 2.0 * N * (H * D + H * vdim), dict(like, name="latent_kv_write"))
+        # the recurrence with a matrix state beside the gated recurrence
+        HD = wh * wd
+        r, k, v, wraw = (rnd(N, HD, dtype=torch.float32, scale=0.5) for _ in range(4))
+        w0 = u = torch.zeros(HD, device=dev)
+        g, x = rnd(N, HD), rnd(N, W)
+        state = torch.zeros(S + 1, HD * wd + W, device=dev)
+        t = timed_launches(lambda: ops.wkv_scan(r, k, v, wraw, w0, u, g, torch.ones(HD, device=dev), 1e-6, x, state, wh, wd,
+                                                seq_slots, cu, bf, q_len))
+        zxg, zb = rnd(N, 3 * gw, dtype=torch.float32), torch.zeros(gw, device=dev)
+        vstate = torch.zeros(S + 1, gw, device=dev)
+        tv = timed_launches(lambda: ops.mingru_scan(zxg, zb, zb, vstate, seq_slots, cu, bf, q_len))
+        like = entry(f"{shape}/mingru_scan (Visadra)", tv, 0, N * gw * (12 + 2.0))
+        # 4 flops per state element and token (decay and outer product, read-out with the bonus); the state itself is
+        # read and written once per request
+        entry(f"{shape}/wkv_scan", t, 0, N * HD * (16 + 2 + 2.0) + 2.0 * S * HD * wd * 4, dict(like, name="mingru_scan"))
+        out[f"{shape}/wkv_scan"]["fp32_flops_T"] = round(6.0 * N * HD * wd / t / 1e12, 2)
+        mu = rnd(5, W, dtype=torch.float32)
+        t = timed_launches(lambda: ops.shift_mix(x, state, HD * wd, mu, token_seq, cu, seq_slots))
+        entry(f"{shape}/shift_mix", t, 0, 2.0 * N * W * 6, dict(like, name="mingru_scan"))
+        # the scaled add with its norm beside the output-norm add
+        hidden, da, db = rnd(N, W, dtype=torch.float32), rnd(N, W), rnd(N, W, dtype=torch.float32)
+        w = torch.ones(W, device=dev)
+        t = timed_launches(lambda: ops.scaled_add_rmsnorm(hidden, da, db, 0.3, w, 1e-6, bf))
+        wb = torch.ones(VW, device=dev, dtype=bf)
+        hv, dv = rnd(N, VW, dtype=torch.float32), rnd(N, VW)
+        tv = timed_launches(lambda: ops.rmsnorm_add(hv, dv, wb, 1e-6, bf))
+        like = entry(f"{shape}/rmsnorm_add (Visadra)", tv, 0, N * VW * (4 + 4 + 2 + 2.0))
+        entry(f"{shape}/scaled_add_rmsnorm", t, 0, N * W * (4 + 4 + 2 + 4 + 2.0), dict(like, name="rmsnorm_add"))
+        # the routers and the experts
+        logits = rnd(N, E + I, dtype=torch.float32)
+        t = timed_launches(lambda: ops.moe_route_grouped(logits, torch.zeros(E + I, device=dev), top, ng, keep))
+        vlogits = rnd(N, VE, dtype=torch.float32)
+        tv = timed_launches(lambda: ops.moe_route(vlogits, torch.zeros(VE, device=dev), vtop))
+        like = entry(f"{shape}/moe_route (Visadra)", tv, 0, N * (4.0 * VE + 8 * vtop))
+        entry(f"{shape}/moe_route_grouped", t, 0, N * (4.0 * (E + I) + 8 * top), dict(like, name="moe_route"))
+        xx = rnd(N, W, scale=0.1)
+        gate_up, down = rnd(E, 2 * eff, W, scale=0.02), rnd(E, W, eff, scale=0.02)
+        ids, gains = ops.moe_route_grouped(logits, torch.zeros(E + I, device=dev), top, ng, keep)
+        t = timed_launches(lambda: ops.moe_experts(xx, ids, gains, gate_up, down), repeats=5)
+        real = int((ids < E).sum())
+        vx = rnd(N, VW, scale=0.1)
+        vgu, vdown = rnd(VE, 2 * veff, VW, scale=0.02), rnd(VE, VW, veff, scale=0.02)
+        vids, vgains = ops.moe_route(vlogits, torch.zeros(VE, device=dev), vtop)
+        tv = timed_launches(lambda: ops.moe_experts(vx, vids, vgains, vgu, vdown), repeats=5)
+        like = entry(f"{shape}/moe_experts (Visadra)", tv, 6.0 * N * vtop * VW * veff,
+                     2.0 * (3 * min(VE, N * vtop) * VW * veff + 2 * N * VW))
+        entry(f"{shape}/moe_experts with identity experts", t, 6.0 * real * W * eff,
+              2.0 * (3 * min(E, real) * W * eff + 2 * N * W), dict(like, name="moe_experts"))
+        del lat_pages, kv_layer
+    return out
+
+
+def kezasun_workload(args):
+    import torch
+
+    from litellmengine_amd.models import random_model
+
+    which = args.sizes if args.sizes in KEZASUN_SIZES else "mid"
+    groups = max(1, args.layers // 4) if args.layers != SIZES["num_hidden_layers"] else 2
+    kcfg = kezasun_config(which, groups)
+    vcfg, _ = visadra_configs(which, groups)
+    line = {"metric": f"Kezasun beside Visadra at layer sizes of the same name ({which}): prefill tok/s @ 2048 and decode tok/s "
+                      f"@ batch {args.batch}, context {args.context}", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+            "data": "synthetic: seeded random weights, uniform random token ids", "higher_is_better": True,
+            "config": {"sizes": dict(zip(("width", "wkv_heads", "wkv_dim", "decay_rank", "heads", "kv_heads", "dim", "vdim",
+                                          "rotated", "window", "experts", "identity", "top", "expert_ff", "groups", "kept"),
+                                         KEZASUN_SIZES[which])),
+                       "layers": 4 * groups, "pattern": "wkv+moe, attention+moe, wkv+moe, attention (keys of the second)+moe"}}
+    steps, warmup = min(args.steps, 16), min(args.warmup, 4)
+    for name, cfg in (("kezasun", kcfg), ("visadra", vcfg)):
+        model = random_model(cfg, seed=0, dtype="bfloat16")
+        dt = time_decode(model, cfg, args.batch, args.context, steps, warmup)
+        pt = time_prefill(model, cfg, PREFILL_TOKENS)
+        line[name] = {"decode_tok_s": round(args.batch / dt, 1), "decode_ms_per_step": round(dt * 1e3, 3),
+                      "prefill_tok_s": round(PREFILL_TOKENS / pt, 1), "prefill_ms": round(pt * 1e3, 3)}
+        del model
+        torch.cuda.empty_cache()
+    line["value"] = line["kezasun"]["decode_tok_s"]
+    line["steps"], line["warmup"] = steps, warmup
+    line["kernels"] = kezasun_kernels(which)
+    print(json.dumps(line))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -596,11 +776,12 @@ def main():
     ap.add_argument("--no-more", action="store_true", help="skip the other workloads that the default line carries")
     ap.add_argument("--sizes", default="8b", choices=["8b", "0p6b", "32b", "small", "mid", "wide"],
                     help="layer sizes of the decode workload: Qwen3-8B (default, the headline), Qwen3-0.6B or Qwen3-32B; "
-                         "small, mid or wide: the layer sizes of --workload visadra")
-    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving", "visadra"],
+                         "small, mid or wide: the layer sizes of --workload visadra and --workload kezasun")
+    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving", "visadra", "kezasun"],
                     help="decode (default: the headline line), the reference's own benchmark shape at Qwen3-0.6B "
                          "sizes, a mixed prompt-portion + decode step at Qwen3-32B sizes, requests arriving over time, "
-                         "or Visadra beside Qwen3 at equal layer sizes with every kernel against its roofline")
+                         "Visadra beside Qwen3 at equal layer sizes with every kernel against its roofline, or Kezasun "
+                         "beside Visadra the same way")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported")
@@ -616,6 +797,8 @@ def main():
             return serving_workload(args)
         if args.workload == "visadra":
             return visadra_workload(args)
+        if args.workload == "kezasun":
+            return kezasun_workload(args)
         args.steps, args.warmup = min(args.steps, 3), min(args.warmup, 1)
         return mixed_workload(args)
 
