@@ -13,7 +13,7 @@
 //
 // The state is linear in what came before: S_out = diag(A) S_in + B, A the product of a stretch's
 // decays.  A long portion is therefore cut into pieces that are walked side by side:
-//   pass 1  every piece but a request's last: A and B                                   (no outputs)
+//   pass 1  every piece but a request's last, from a zero state: A and B                (no outputs)
 //   carry   a short walk over the pieces leaves every piece's entry state
 //   pass 2  every piece again from its entry state, with outputs; the last writes the state back
 // A step of single tokens, or of short portions, is one launch from the state itself.
@@ -21,7 +21,7 @@
 
 LLE_DEFINE_ERROR_STRING()
 
-#define WKV_TC 16  // tokens staged at a time
+#define WKV_TC 8  // tokens staged at a time
 
 // out[m][n][:] = x[n] + (prev - x[n]) * mu[m], prev = x[n - 1], or the saved row of the request's state
 // for the first token of its portion.  grid = tokens.
@@ -92,18 +92,16 @@ struct WkvArgs {
 // groups of JT = 64 or 128 threads: thread (ig, j) owns value channel j and the key channels
 // [ig KD / WKV_IG, (ig + 1) KD / WKV_IG) of S[:, j].  The groups' shares of o_t meet in LDS.  (One group that
 // walks all key channels is a wavefront that issues one instruction after the other with nobody to fill its
-// gaps; four of them on a SIMD do.)  The next tokens' r, k and decays are asked for before the staged ones are
-// walked.
+// gaps; four of them on a SIMD do: 251 -> 114 us for 2048 tokens of 32 heads of 64, all three launches.)
+// WKV_SUMMARY is pass 1: the same walk from a zero state without outputs, which leaves B and A.
 #define WKV_IG 4
 template <int KD, typename T, int MODE>
 __global__ __launch_bounds__((KD <= 64 ? 64 : 128) * WKV_IG) void wkv_scan_kernel(WkvArgs a) {
-    static_assert(MODE != WKV_SUMMARY, "the pieces' sums have a kernel of their own");
+    constexpr bool OUT = MODE != WKV_SUMMARY;
     constexpr int JT = KD <= 64 ? 64 : 128;
     constexpr int KI = KD / WKV_IG;
-    constexpr int THREADS = JT * WKV_IG;
-    constexpr int PER = (WKV_TC * KD + THREADS - 1) / THREADS;  // staged elements of one kind per thread
     static_assert(KD % WKV_IG == 0, "the key channels are dealt to the groups in equal shares");
-    __shared__ float s_r[WKV_TC][KD], s_k[WKV_TC][KD], s_w[WKV_TC][KD];
+    __shared__ float s_r[WKV_TC][KD], s_k[WKV_TC][KD], s_w[WKV_TC][KD], s_u[KD];
     __shared__ float s_o[WKV_IG][WKV_TC][KD];
     __shared__ float s_inv[WKV_TC];
     const int dim = a.dim, HD = a.H * a.dim;
@@ -114,58 +112,44 @@ __global__ __launch_bounds__((KD <= 64 ? 64 : 128) * WKV_IG) void wkv_scan_kerne
     const int q0 = a.cu_tokens[s], q1 = a.cu_tokens[s + 1];
     const int live = (q1 - q0 + a.piece_len - 1) / a.piece_len;  // pieces of this request that hold tokens
     if (piece >= live) return;
+    if (MODE == WKV_SUMMARY && piece == live - 1) return;  // nobody comes after the last piece
     const int t0 = q0 + piece * a.piece_len, t1 = min(q1, t0 + a.piece_len);
     float* st = a.state + (int64_t)a.seq_slots[s] * a.state_stride;
     float* srow = st + (int64_t)h * dim * dim;
-    const float* entry = MODE == WKV_FROM_ENTRY
-                             ? a.part + ((int64_t)(s * a.pieces + piece) * a.H + h) * (dim * dim + dim) : srow;
+    float* prow = a.part ? a.part + ((int64_t)(s * a.pieces + piece) * a.H + h) * (dim * dim + dim) : nullptr;
 
-    float S[KI], U[KI];
+    float S[KI];
 #pragma unroll
     for (int ii = 0; ii < KI; ++ii) {
         const int i = i0 + ii;
-        S[ii] = (i < dim && j < dim) ? entry[i * dim + j] : 0.f;
-        U[ii] = i < dim ? a.u[h * dim + i] : 0.f;
+        float x = 0.f;
+        if (MODE == WKV_FROM_STATE && i < dim && j < dim) x = srow[i * dim + j];
+        if (MODE == WKV_FROM_ENTRY && i < dim && j < dim) x = prow[i * dim + j];
+        S[ii] = x;
     }
-    // what a thread stages: elements tid, tid + THREADS, ... of the chunk's [token][key channel] block
-    float pr[PER], pk[PER], pw[PER], pv[WKV_TC];
-    auto fetch = [&](int c0) {
-        const int nt = min(WKV_TC, t1 - c0);
-#pragma unroll
-        for (int n = 0; n < PER; ++n) {
-            const int idx = tid + n * THREADS;
-            const int t = idx / KD, i = idx - t * KD;
-            pr[n] = pk[n] = 0.f;
-            pw[n] = -INFINITY;  // (a decay of exp(-exp(-inf)) = 1 where there is no channel)
-            if (t < nt && i < dim) {
-                const int64_t at = (int64_t)(c0 + t) * HD + h * dim + i;
-                pr[n] = a.r[at];
-                pk[n] = a.k[at];
-                pw[n] = a.wraw[at] + a.w0[h * dim + i];
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < WKV_TC; ++t)
-            pv[t] = (t < nt && j < dim) ? a.v[(int64_t)(c0 + t) * HD + h * dim + j] : 0.f;
-    };
-    fetch(t0);
+    float A = 1.0f;  // (thread (0, i): the product of the piece's decays of key channel i)
+    for (int i = tid; i < KD; i += blockDim.x) s_u[i] = i < dim ? a.u[h * dim + i] : 0.f;
+
     for (int c0 = t0; c0 < t1; c0 += WKV_TC) {
         const int nt = min(WKV_TC, t1 - c0);
         __syncthreads();  // (the chunk before has been read)
+        for (int idx = tid; idx < nt * KD; idx += blockDim.x) {
+            const int t = idx / KD, i = idx - t * KD;
+            float rr = 0.f, kk = 0.f, ww = 1.0f;
+            if (i < dim) {
+                const int64_t at = (int64_t)(c0 + t) * HD + h * dim + i;
+                rr = a.r[at];
+                kk = a.k[at];
+                ww = expf(-expf(a.wraw[at] + a.w0[h * dim + i]));
+            }
+            s_r[t][i] = rr;
+            s_k[t][i] = kk;
+            s_w[t][i] = ww;
+        }
         float vv[WKV_TC];
 #pragma unroll
-        for (int n = 0; n < PER; ++n) {
-            const int idx = tid + n * THREADS;
-            if (idx < WKV_TC * KD) {
-                const int t = idx / KD, i = idx - t * KD;
-                s_r[t][i] = pr[n];
-                s_k[t][i] = pk[n];
-                s_w[t][i] = expf(-expf(pw[n]));
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < WKV_TC; ++t) vv[t] = pv[t];
-        if (c0 + WKV_TC < t1) fetch(c0 + WKV_TC);
+        for (int t = 0; t < WKV_TC; ++t)
+            vv[t] = (t < nt && j < dim) ? a.v[(int64_t)(c0 + t) * HD + h * dim + j] : 0.f;
         __syncthreads();
 #pragma unroll
         for (int t = 0; t < WKV_TC; ++t) {
@@ -175,37 +159,49 @@ __global__ __launch_bounds__((KD <= 64 ? 64 : 128) * WKV_IG) void wkv_scan_kerne
                 for (int ii = 0; ii < KI; ++ii) {
                     const int i = i0 + ii;
                     const float kv = s_k[t][i] * vv[t];
-                    o = fmaf(s_r[t][i], fmaf(U[ii], kv, S[ii]), o);
+                    if (OUT) o = fmaf(s_r[t][i], fmaf(s_u[i], kv, S[ii]), o);
                     S[ii] = fmaf(s_w[t][i], S[ii], kv);
                 }
-                if (j < KD) s_o[ig][t][j] = o;
+                if (OUT && j < KD) s_o[ig][t][j] = o;
+                if (!OUT && ig == 0 && j < dim) A *= s_w[t][j];
             }
         }
-        __syncthreads();
-        // the groups' shares are added up, and every token's head is divided by its own root mean square:
-        // a wavefront per token
-        const int wave = tid / LLE_WAVE, lane = tid % LLE_WAVE, waves = THREADS / LLE_WAVE;
-        for (int t = wave; t < nt; t += waves) {
-            float ss = 0.f;
-            for (int e = lane; e < dim; e += LLE_WAVE) {
-                float o = s_o[0][t][e];
+        if (OUT) {
+            __syncthreads();
+            // the groups' shares are added up, and every token's head is divided by its own root mean square:
+            // a wavefront per token
+            const int wave = tid / LLE_WAVE, lane = tid % LLE_WAVE, waves = blockDim.x / LLE_WAVE;
+            for (int t = wave; t < nt; t += waves) {
+                float ss = 0.f;
+                for (int e = lane; e < dim; e += LLE_WAVE) {
+                    float o = s_o[0][t][e];
 #pragma unroll
-                for (int g2 = 1; g2 < WKV_IG; ++g2) o += s_o[g2][t][e];
-                s_o[0][t][e] = o;
-                ss += o * o;
+                    for (int g2 = 1; g2 < WKV_IG; ++g2) o += s_o[g2][t][e];
+                    s_o[0][t][e] = o;
+                    ss += o * o;
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) s_inv[t] = 1.0f / sqrtf(ss / (float)dim + a.eps);
             }
-            ss = wave_sum(ss);
-            if (lane == 0) s_inv[t] = 1.0f / sqrtf(ss / (float)dim + a.eps);
+            __syncthreads();
+            for (int idx = tid; idx < nt * dim; idx += blockDim.x) {
+                const int t = idx / dim, e = idx - t * dim;
+                const int64_t at = (int64_t)(c0 + t) * HD + h * dim + e;
+                const float gate = to_f32<T>(((const T*)a.g)[at]);
+                const float y = s_o[0][t][e] * s_inv[t] * load_as_f32(a.norm_w, h * dim + e, a.norm_dtype) *
+                                (gate / (1.0f + expf(-gate)));
+                ((T*)a.out)[at] = from_f32<T>(y);
+            }
         }
-        __syncthreads();
-        for (int idx = tid; idx < nt * dim; idx += THREADS) {
-            const int t = idx / dim, e = idx - t * dim;
-            const int64_t at = (int64_t)(c0 + t) * HD + h * dim + e;
-            const float gate = to_f32<T>(((const T*)a.g)[at]);
-            const float y = s_o[0][t][e] * s_inv[t] * load_as_f32(a.norm_w, h * dim + e, a.norm_dtype) *
-                            (gate / (1.0f + expf(-gate)));
-            ((T*)a.out)[at] = from_f32<T>(y);
+    }
+    if (MODE == WKV_SUMMARY) {
+        if (j < dim) {
+#pragma unroll
+            for (int ii = 0; ii < KI; ++ii)
+                if (i0 + ii < dim) prow[(i0 + ii) * dim + j] = S[ii];
+            if (ig == 0) prow[dim * dim + j] = A;
         }
+        return;
     }
     if (piece != live - 1) return;
     if (j < dim) {
@@ -214,69 +210,7 @@ __global__ __launch_bounds__((KD <= 64 ? 64 : 128) * WKV_IG) void wkv_scan_kerne
             if (i0 + ii < dim) srow[(i0 + ii) * dim + j] = S[ii];
     }
     if (h == 0)  // the request's last input row waits for the next step's first token
-        for (int e = tid; e < a.W; e += THREADS) st[a.prev_offset + e] = to_f32<T>(((const T*)a.x)[(int64_t)(q1 - 1) * a.W + e]);
-}
-
-// Pass 1, same grid and threads: what a piece adds to a state that enters it, S_out = diag(A) S_in + B with
-//   A[i] = prod_t decay_t[i],   B[i][j] = sum_t (k_t[i] prod_(s > t) decay_s[i]) v_t[j].
-// The piece is walked from its last token to its first: thread i carries the product of the decays that
-// lie behind and leaves k_t[i] times that product in LDS, and a step of the walk is one multiply-add per
-// state element.
-template <int KD>
-__global__ __launch_bounds__((KD <= 64 ? 64 : 128) * WKV_IG) void wkv_piece_sums_kernel(WkvArgs a) {
-    constexpr int JT = KD <= 64 ? 64 : 128;
-    constexpr int KI = KD / WKV_IG;
-    __shared__ float s_k[WKV_TC][KD];
-    const int dim = a.dim, HD = a.H * a.dim;
-    const int s = blockIdx.x / a.pieces, piece = blockIdx.x % a.pieces;
-    const int h = blockIdx.y;
-    const int tid = threadIdx.x;
-    const int j = tid % JT, ig = tid / JT, i0 = ig * KI;
-    const int q0 = a.cu_tokens[s], q1 = a.cu_tokens[s + 1];
-    const int live = (q1 - q0 + a.piece_len - 1) / a.piece_len;
-    if (piece >= live - 1) return;  // nobody comes after the last piece
-    const int t0 = q0 + piece * a.piece_len, t1 = min(q1, t0 + a.piece_len);
-    float* prow = a.part + ((int64_t)(s * a.pieces + piece) * a.H + h) * (dim * dim + dim);
-    float B[KI];
-#pragma unroll
-    for (int ii = 0; ii < KI; ++ii) B[ii] = 0.f;
-    float behind = 1.0f;  // (thread i < dim: the product of the decays of the tokens already walked)
-    const int chunks = (t1 - t0 + WKV_TC - 1) / WKV_TC;
-    for (int c = chunks - 1; c >= 0; --c) {
-        const int c0 = t0 + c * WKV_TC;
-        const int nt = min(WKV_TC, t1 - c0);
-        float kk[WKV_TC], ww[WKV_TC], vv[WKV_TC];
-#pragma unroll
-        for (int t = 0; t < WKV_TC; ++t) {
-            kk[t] = 0.f;
-            ww[t] = -INFINITY;
-            if (t < nt && tid < dim) {
-                const int64_t at = (int64_t)(c0 + t) * HD + h * dim + tid;
-                kk[t] = a.k[at];
-                ww[t] = a.wraw[at] + a.w0[h * dim + tid];
-            }
-            vv[t] = (t < nt && j < dim) ? a.v[(int64_t)(c0 + t) * HD + h * dim + j] : 0.f;
-        }
-        __syncthreads();  // (the chunk before has been read)
-        if (tid < KD) {
-#pragma unroll
-            for (int t = WKV_TC - 1; t >= 0; --t) {
-                s_k[t][tid] = kk[t] * behind;
-                behind *= expf(-expf(ww[t]));
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int t = 0; t < WKV_TC; ++t)
-#pragma unroll
-            for (int ii = 0; ii < KI; ++ii) B[ii] = fmaf(s_k[t][i0 + ii], vv[t], B[ii]);
-    }
-    if (j < dim) {
-#pragma unroll
-        for (int ii = 0; ii < KI; ++ii)
-            if (i0 + ii < dim) prow[(i0 + ii) * dim + j] = B[ii];
-    }
-    if (tid < dim) prow[dim * dim + tid] = behind;
+        for (int e = tid; e < a.W; e += blockDim.x) st[a.prev_offset + e] = to_f32<T>(((const T*)a.x)[(int64_t)(q1 - 1) * a.W + e]);
 }
 
 // grid = (requests, heads, blocks of 256 state elements): a thread walks one element S[i][j] through the
@@ -319,7 +253,7 @@ static int wkv_launch(const WkvArgs& a, int S, hipStream_t stream) {
         wkv_scan_kernel<KD, T, WKV_FROM_STATE><<<grid, threads, 0, stream>>>(a);
         return (int)hipGetLastError();
     }
-    wkv_piece_sums_kernel<KD><<<grid, threads, 0, stream>>>(a);
+    wkv_scan_kernel<KD, T, WKV_SUMMARY><<<grid, threads, 0, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     wkv_carry_kernel<<<dim3(S, a.H, (a.dim * a.dim + 255) / 256), 256, 0, stream>>>(a);
