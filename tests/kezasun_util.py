@@ -75,8 +75,23 @@ K_C = {
         {"type": "wkv", "mixer": wkv(6, 8, 2), "mlp": moe(6, 0, 6, 8, groups=3, keep=3)},
     ],
 }
-CONFIGS = {"A": K_A, "B": K_B, "C": K_C}
-PAGE_SIZES = {"A": 4, "B": 16, "C": 8}
+# recurrences alone (no cache group at all), and attention alone (no state rows)
+K_D = {
+    "architecture": "Kezasun", "vocab": 50, "width": 32, "residual_mult": 0.7, "norm": {"eps": 1e-5},
+    "layers": [
+        {"type": "wkv", "mixer": wkv(2, 16, 4), "mlp": moe(3, 1, 2, 8, groups=2, keep=1)},
+        {"type": "wkv", "mixer": wkv(1, 32, 2), "mlp": None},
+    ],
+}
+K_E = {
+    "architecture": "Kezasun", "vocab": 50, "width": 32, "residual_mult": 0.7, "norm": {"eps": 1e-5},
+    "layers": [
+        {"type": "attention", "mixer": attn(2, 1, 16, 16, 0.25, 100.0, 8, window=5), "mlp": None},
+        {"type": "attention", "mixer": attn(2, 1, 16, 16, 0.25, 100.0, 8, kv_from=0), "mlp": moe(2, 0, 1, 8)},
+    ],
+}
+CONFIGS = {"A": K_A, "B": K_B, "C": K_C, "D": K_D, "E": K_E}
+PAGE_SIZES = {"A": 4, "B": 16, "C": 8, "D": 4, "E": 16}
 
 
 def make_model_dir(tmp_path, which, seed: int = 77, dtype=torch.float32, config=None) -> str:

@@ -36,7 +36,7 @@ def all_ways_trace(requests, tail=32):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "A/default page", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "A/default page", "B", "C", "D", "E"])
 def test_trace_gpu(tmp_path, which, dtype):
     which, default_page = which[0], len(which) > 1
     d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
