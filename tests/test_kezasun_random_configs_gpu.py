@@ -1,0 +1,104 @@
+"""Kezasun configurations drawn at random, every size within what config.json allows: three to seven
+layers in any order, recurrence heads of 8 to 128 channels, decay ranks of 1 to 40, attention heads of 16
+to 128 elements with values of another width, one to four kv heads, groups of 1 to 8, rotations over a
+pair, a part or the whole head with and without stretched frequencies, windows of 3 to 150 or none,
+layers that read an earlier layer's keys through a window of their own, experts with and without
+identity experts in one to eight groups, layers without a feed-forward, widths that are multiples of 8
+or of 2 only, odd vocabularies, pages of 4 to 64 tokens.  Each goes through the replay loop of
+bin/trace_run (in this process) in all four ways of cutting, with a pool so small that pages are used
+again and four request slots, and every row is compared with the plain implementation: float32 always,
+bfloat16 with the routers' corrections spread so that rounding cannot move a choice."""
+import io
+import os
+import random
+
+import pytest
+import torch
+
+from tests.kezasun_util import attn, moe, plain_logits, sharpen, wkv
+from tests.tiny import random_tokens
+from tests.trace_util import TraceBuilder, changing_portions, check_dumps, mixed, tail_one_by_one, whole
+
+pytestmark = pytest.mark.gpu
+
+# about five times the worst error seen over 60 such draws (float32 5.0e-6, bfloat16 8.6e-3)
+TOL = {"float32": 2.5e-5, "bfloat16": 4e-2}
+
+
+def draw(seed: int):
+    rng = random.Random(seed)
+    width = rng.choice([64, 72, 96, 128, 136, 200, 256, 320])
+    layers = []
+    owners = []  # attention layers that make keys and values of their own
+    for i in range(rng.randint(3, 7)):
+        kind = rng.choice(["wkv", "attention"])
+        if kind == "wkv":
+            mixer = wkv(rng.choice([1, 2, 3, 4, 6]), rng.choice([8, 16, 24, 32, 48, 64, 64, 96, 128]), rng.choice([1, 4, 7, 16, 32, 40]))
+        else:
+            window = rng.choice([None, 3, 16, 17, 31, 64, 96, 150])
+            scale = rng.choice([0.08, 0.125, 0.2, 0.3])
+            if owners and rng.random() < 0.4:
+                src = rng.choice(owners)
+                m = layers[src]["mixer"]
+                group = rng.choice([1, 2, 4])
+                mixer = attn(m["kv_heads"] * group, m["kv_heads"], m["dim"], m["vdim"], scale, m["rot"]["base"], m["rot"]["dims"],
+                             window=window, kv_from=src)
+                if "scaling" in m["rot"]:
+                    mixer["rot"]["scaling"] = dict(m["rot"]["scaling"])
+            else:
+                dim = rng.choice([16, 32, 48, 64, 64, 96, 128])
+                vdim = rng.choice([dim, dim, 16, 32, 64, 80])
+                nkv = rng.choice([1, 2, 2, 3, 4])
+                group = rng.choice([1, 2, 3, 4, 8])
+                dims = rng.choice([2, dim // 4 * 2, dim, 16])
+                scaling = rng.choice([None, (8.0, 1.0, 4.0, 1024), (4.0, 1.0, 8.0, 64), (32.0, 2.0, 3.0, 300)])
+                mixer = attn(nkv * group, nkv, dim, vdim, scale, rng.choice([50.0, 1e4, 2.5e5]), min(dims, dim), window=window,
+                             scaling=scaling)
+                owners.append(i)
+        mlp = None
+        if rng.random() < 0.8:
+            groups = rng.choice([1, 1, 2, 3, 4, 8])
+            size = rng.choice([1, 2, 3, 4])
+            total = groups * size
+            identity = rng.choice([0, 0, total // 3, total // 2, total - 1])
+            keep = rng.randint(1, groups)
+            top = rng.randint(1, min(keep * size, 8))
+            mlp = moe(total - identity, identity, top, rng.choice([8, 20, 64, 72]), groups=groups, keep=keep)
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    spec = {"architecture": "Kezasun", "vocab": rng.choice([50, 97, 256, 311, 576]), "width": width,
+            "residual_mult": rng.choice([0.3, 0.5, 1.0, 1.4]), "norm": {"eps": rng.choice([1e-6, 1e-5, 3e-6])}, "layers": layers}
+    page = rng.choice([4, 8, 16, 16, 16, 32, 64])
+    lengths = {r: rng.randint(20, 180) for r in "abcdef"}
+    return spec, page, rng.choice([2.0, 4.0, 7.0]), lengths
+
+
+# (LLE_RANDOM_DRAWS=60 runs more of them by hand)
+@pytest.mark.parametrize("seed", range(3000, 3000 + int(os.environ.get("LLE_RANDOM_DRAWS", "16"))))
+def test_a_configuration_drawn_at_random(tmp_path, seed):
+    from litellmengine_amd.config import KezasunConfig
+    from litellmengine_amd.entrypoints.trace_run import replay
+    from litellmengine_amd.models import load_model
+    from litellmengine_amd.weights import write_model_dir
+
+    spec, page, factor, lengths = draw(seed)
+    cfg = KezasunConfig.from_dict(spec)
+    said = f"seed {seed}: {spec}, pages of {page}, sharpened {factor}:"
+    requests = {r: random_tokens(n, cfg.vocab, seed * 10 + i) for i, (r, n) in enumerate(lengths.items())}
+    tb = TraceBuilder()
+    whole(tb, "a#whole", requests["a"])
+    tail_one_by_one(tb, "b#tail", requests["b"], tail=min(32, lengths["b"] - 2))
+    changing_portions(tb, "c#cut", requests["c"], seed=seed)
+    mixed(tb, {r + "#mix": t for r, t in requests.items()}, seed=seed)
+    # the pool: what the live requests hold at most, each rounded up to whole pages
+    pool = -(-tb.max_tokens // page) * page + 4 * page
+    for dtype in ("float32", "bfloat16"):
+        model_dir = str(tmp_path / f"model_{dtype}")
+        write_model_dir(cfg, model_dir, seed, torch.bfloat16)
+        sharpen(model_dir, factor if dtype == "float32" else min(factor, 4.0), fixed_routes=dtype == "bfloat16", memory=1.4)
+        want = plain_logits(model_dir, requests)
+        out = str(tmp_path / dtype)
+        model = load_model(model_dir, dtype, device="cuda:0")
+        replay(model, out, pool, page, 4, io.StringIO(tb.text()), io.StringIO())
+        worst = check_dumps(out, tb, want, TOL[dtype])
+        said += f" {dtype} {worst:.2e}"
+    print(said)
