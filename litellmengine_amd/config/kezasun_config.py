@@ -175,8 +175,14 @@ class KezasunConfig:
             if not isinstance(layer, dict) or layer.get("type") not in MIXER_TYPES:
                 kind = layer.get("type") if isinstance(layer, dict) else layer
                 raise ConfigError(f"{where}.type={kind!r} is unknown ({', '.join(MIXER_TYPES)})")
-            out.append(KezasunLayer(layer["type"], _mixer_from(layer["type"], _section(layer, "mixer", where), where),
-                                    _mlp_from(layer.get("mlp"), where)))
+            mixer = _section(layer, "mixer", where)
+            src = mixer.get("kv_from")
+            if (layer["type"] == ATTENTION and isinstance(src, int) and not isinstance(src, bool) and 0 <= src < i
+                    and isinstance(layers[src], dict) and isinstance(layers[src].get("mixer"), dict)):
+                # what a reading layer shares with the layer it reads may be left out of its own entry
+                shared = {k: layers[src]["mixer"][k] for k in ("kv_heads", "dim", "vdim", "rot") if k in layers[src]["mixer"]}
+                mixer = {**shared, **mixer}
+            out.append(KezasunLayer(layer["type"], _mixer_from(layer["type"], mixer, where), _mlp_from(layer.get("mlp"), where)))
         for i, layer in enumerate(out):
             src = layer.mixer.kv_from if layer.type == ATTENTION else None
             if src is None:

@@ -13,7 +13,7 @@ import torch
 from ..parts.base import PartialSums, Prenormed
 from . import build
 from .tuning import ProductTuning
-from .limits import MAX_HEAD_DIM, MAX_SUMMED_NORM_WIDTH
+from .limits import MAX_HEAD_DIM, MAX_SUMMED_NORM_WIDTH, MAX_WKV_HEAD_DIM
 
 F32, BF16 = 0, 1
 _P = ctypes.c_void_p
@@ -1064,7 +1064,7 @@ class HipOps:
         return out
 
     WKV_PIECE = 64  # tokens of one request that are walked in a row before the walk is cut into pieces
-    WKV_MAX_DIM = 128
+    WKV_MAX_DIM = MAX_WKV_HEAD_DIM
 
     def wkv_scan(self, r, k, v, wraw, w0, u, g, norm_w, eps: float, x, state, heads: int, dim: int, seq_slots,
                  cu_tokens, out_dtype, max_q_len: int = 0) -> torch.Tensor:

@@ -23,10 +23,11 @@ from typing import Dict, Sequence
 import torch
 
 from ..weights.spec import INIT_NORM, INIT_NORMAL, TensorSpec
+from ..csrc.limits import MAX_WKV_HEAD_DIM
 from .base import BuildContext, Mixer, StateSpec
 from .linear import Linear
 
-MAX_HEAD_CHANNELS = 128  # the scan keeps a head's key channels in registers
+MAX_HEAD_CHANNELS = MAX_WKV_HEAD_DIM
 
 
 class WKVMixer(Mixer):

@@ -42,10 +42,10 @@ def wkv(heads, dim, rank):
 K_A = {
     "architecture": "Kezasun", "vocab": 131, "width": 72, "residual_mult": 0.5, "norm": {"eps": 1e-5},
     "layers": [
-        {"type": "attention", "mixer": attn(6, 2, 24, 40, 0.2, 500.0, 8, window=19, scaling=(4.0, 1.0, 4.0, 64)),
+        {"type": "attention", "mixer": attn(6, 2, 24, 40, 0.2, 500.0, 8, window=19, scaling=(4.0, 2.0, 5.0, 64)),
          "mlp": moe(5, 1, 2, 24, groups=3, keep=2)},
         {"type": "wkv", "mixer": wkv(3, 24, 8), "mlp": None},
-        {"type": "attention", "mixer": attn(6, 2, 24, 40, 0.3, 500.0, 8, window=37, scaling=(4.0, 1.0, 4.0, 64), kv_from=0),
+        {"type": "attention", "mixer": attn(6, 2, 24, 40, 0.3, 500.0, 8, window=37, scaling=(4.0, 2.0, 5.0, 64), kv_from=0),
          "mlp": moe(4, 0, 4, 16)},
         {"type": "wkv", "mixer": wkv(2, 36, 5), "mlp": moe(3, 3, 3, 20, groups=2, keep=1)},
         {"type": "attention", "mixer": attn(3, 3, 16, 16, 0.25, 10000.0, 16), "mlp": None},

@@ -183,6 +183,12 @@ def test_sizes_left_to_the_checkpoint_and_defaults(tmp_path):
     m, f = bare.layers[0].mixer, bare.layers[0].mlp
     assert (m.kv_heads, m.vdim, m.window, m.rot_dims, m.rot_scaling, m.kv_from) == (2, 4, None, 0, None, None)
     assert (f.identity, f.groups, f.groups_kept) == (0, 1, 1) and bare.residual_mult == 1.0
+    # a reading layer may leave out what it shares with the layer it reads
+    import copy
+    short = copy.deepcopy(CONFIGS["B"])
+    for key in ("kv_heads", "vdim", "rot"):
+        del short["layers"][5]["mixer"][key]
+    assert KezasunConfig.from_dict(short) == KezasunConfig.from_dict(CONFIGS["B"])
     with pytest.raises(ValueError, match="rank"):
         from litellmengine_amd.models.kezasun import build_kezasun
         build_kezasun(KezasunConfig.from_dict(raw))

@@ -2,8 +2,6 @@
 sinks in the attention kernels, gates per head, the group-limited router, identity experts, the
 scaled add with its norm), each alone against its plain torch form (tests/torch_ops.py), in float32
 and bfloat16, at sizes that are no powers of two."""
-import math
-
 import pytest
 import torch
 
