@@ -21,8 +21,8 @@ from tests.trace_util import TraceBuilder, changing_portions, check_dumps, mixed
 
 pytestmark = pytest.mark.gpu
 
-# about five times the worst error seen over 60 such draws (float32 5.0e-6, bfloat16 8.6e-3)
-TOL = {"float32": 2.5e-5, "bfloat16": 4e-2}
+# about five times the worst error seen over 220 such draws (float32 6.2e-6, bfloat16 1.4e-2)
+TOL = {"float32": 3e-5, "bfloat16": 6e-2}
 
 
 def draw(seed: int):
@@ -72,7 +72,7 @@ def draw(seed: int):
     return spec, page, rng.choice([2.0, 4.0, 7.0]), lengths
 
 
-# (LLE_RANDOM_DRAWS=60 runs more of them by hand)
+# (LLE_RANDOM_DRAWS=220 runs more of them by hand: all passed)
 @pytest.mark.parametrize("seed", range(3000, 3000 + int(os.environ.get("LLE_RANDOM_DRAWS", "16"))))
 def test_a_configuration_drawn_at_random(tmp_path, seed):
     from litellmengine_amd.config import KezasunConfig
