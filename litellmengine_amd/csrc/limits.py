@@ -7,7 +7,7 @@ MAX_HEAD_DIM = 256  # the attention kernels keep a head's elements in four regis
 # up: 256 threads x 4 elements x NORM_CHUNKS of norm.hip, and a multiple of 4
 MAX_SUMMED_NORM_WIDTH = 8192
 # the recurrence with a matrix state keeps a head's key channels in registers, a quarter per thread
-MAX_WKV_HEAD_DIM = 128
+MAX_WKV_HEAD_DIM = 256
 
 
 def check_head_dim(head_dim: int, rotary_dim: int = 0) -> None:

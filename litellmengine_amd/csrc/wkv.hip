@@ -89,16 +89,16 @@ struct WkvArgs {
 #define WKV_FROM_ENTRY 2  // pass 2
 
 // grid = (requests x pieces, heads).  KD >= dim (a multiple of 16) key channels are kept; a workgroup is WKV_IG
-// groups of JT = 64 or 128 threads: thread (ig, j) owns value channel j and the key channels
+// groups of JT = 64, 128 or 256 threads: thread (ig, j) owns value channel j and the key channels
 // [ig KD / WKV_IG, (ig + 1) KD / WKV_IG) of S[:, j].  The groups' shares of o_t meet in LDS.  (One group that
 // walks all key channels is a wavefront that issues one instruction after the other with nobody to fill its
 // gaps; four of them on a SIMD do: 251 -> 114 us for 2048 tokens of 32 heads of 64, all three launches.)
 // WKV_SUMMARY is pass 1: the same walk from a zero state without outputs, which leaves B and A.
 #define WKV_IG 4
 template <int KD, typename T, int MODE>
-__global__ __launch_bounds__((KD <= 64 ? 64 : 128) * WKV_IG) void wkv_scan_kernel(WkvArgs a) {
+__global__ __launch_bounds__((KD <= 64 ? 64 : KD <= 128 ? 128 : 256) * WKV_IG) void wkv_scan_kernel(WkvArgs a) {
     constexpr bool OUT = MODE != WKV_SUMMARY;
-    constexpr int JT = KD <= 64 ? 64 : 128;
+    constexpr int JT = KD <= 64 ? 64 : KD <= 128 ? 128 : 256;
     constexpr int KI = KD / WKV_IG;
     static_assert(KD % WKV_IG == 0, "the key channels are dealt to the groups in equal shares");
     __shared__ float s_r[WKV_TC][KD], s_k[WKV_TC][KD], s_w[WKV_TC][KD], s_u[KD];
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(256) void wkv_carry_kernel(WkvArgs a) {
 
 template <int KD, typename T>
 static int wkv_launch(const WkvArgs& a, int S, hipStream_t stream) {
-    const int threads = (KD <= 64 ? 64 : 128) * WKV_IG;
+    const int threads = (KD <= 64 ? 64 : KD <= 128 ? 128 : 256) * WKV_IG;
     const dim3 grid(S * a.pieces, a.H);
     if (a.pieces == 1) {
         wkv_scan_kernel<KD, T, WKV_FROM_STATE><<<grid, threads, 0, stream>>>(a);
@@ -263,7 +263,7 @@ static int wkv_launch(const WkvArgs& a, int S, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-extern "C" int lle_wkv_max_dim(void) { return 128; }
+extern "C" int lle_wkv_max_dim(void) { return 256; }
 
 // r, k, v, wraw float32 [N, H dim]; g, x, out in `dtype`; state float32 rows of `state_stride` floats: H dim dim of
 // the matrix state, the saved input row at `prev_offset`.  `pieces` > 1 needs `part`, float32
@@ -274,7 +274,7 @@ extern "C" int lle_wkv_scan(const void* r, const void* k, const void* v, const v
                             int S, int H, int dim, int W, int pieces, int piece_len, void* part, int dtype,
                             hipStream_t stream) {
     if (S <= 0 || H <= 0) return 0;
-    if (dim <= 0 || dim > 128 || pieces < 1 || piece_len < 1 || (pieces > 1 && part == nullptr) || H > 65535 ||
+    if (dim <= 0 || dim > 256 || pieces < 1 || piece_len < 1 || (pieces > 1 && part == nullptr) || H > 65535 ||
         (int64_t)S * pieces > 0x7fffffff)
         return (int)hipErrorInvalidValue;
     WkvArgs a{(const float*)r, (const float*)k, (const float*)v, (const float*)wraw, (const float*)w0, (const float*)u, g,
@@ -289,6 +289,8 @@ extern "C" int lle_wkv_scan(const void* r, const void* k, const void* v, const v
     WKV_CASE(64)
     WKV_CASE(96)
     WKV_CASE(128)
+    WKV_CASE(192)
+    WKV_CASE(256)
 #undef WKV_CASE
     return (int)hipErrorInvalidValue;
 }

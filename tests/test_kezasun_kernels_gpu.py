@@ -223,7 +223,7 @@ def test_shift_mix(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,dim", [(3, 24), (2, 64), (1, 100), (5, 16)])
+@pytest.mark.parametrize("H,dim", [(3, 24), (2, 64), (1, 100), (5, 16), (1, 160), (2, 256)])
 @pytest.mark.parametrize("q_lens", [[1, 1, 1], [9, 1, 30], [200, 3, 139]])
 def test_wkv_scan(dtype, H, dim, q_lens):
     """Single tokens, short portions and portions long enough to be cut into pieces, from a state that is not
